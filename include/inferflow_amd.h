@@ -39,7 +39,7 @@ extern "C" {
 #endif
 
 typedef enum {
-    IFA_F32 = 0, IFA_F16 = 1,
+    IFA_F32 = 0, IFA_F16 = 1, IFA_BF16 = 2,
     IFA_Q8_B32T1 = 7, IFA_Q8_B32T2 = 8, IFA_Q6_B64T1 = 9, IFA_Q5_B64T1 = 10, IFA_Q5_B32T1 = 11,
     IFA_Q4_B16 = 12, IFA_Q4_B32T1A = 13, IFA_Q4_B32T1B = 14, IFA_Q4_B64T1 = 17, IFA_Q3H_B64T1 = 18,
     IFA_Q3_B32T1A = 19, IFA_Q3_B32T1B = 20, IFA_Q2_B32T1A = 21, IFA_Q2_B32T1B = 22
@@ -448,6 +448,117 @@ int ifa_model_get_expert_tensor(ifa_model *m, int layer, int expert, int tensor_
  * launches of one fused decode kernel, rotating over the layers' weights:
  * which = 0 qkv, 1 attention, 2 wo, 3 ffn w1/w3, 4 w2, 5 lm_head.  For bench.py's roofline. */
 int ifa_model_time_kernel(ifa_model *m, int which, int iters, float *avg_us);
+
+
+/* ======================================================================== */
+/* Ops on 32-bit activations with bfloat16 parameters (csrc/ifa_linear_bf16.hip, ifa_ops_f32.hip, ifa_seqmix.hip,         */
+/* ifa_attn_window.hip): the building blocks of the layer-list worker below, usable on their own.  Activations, the         */
+/* residual stream, attention scores and every recurrent state are fp32; weights are bfloat16 bit patterns.               */
+/* ======================================================================== */
+/* C[t][n] (+)= alpha * mul[n] * (sum_k A[t][k] W[n][k] + bias[n]);  W bf16 [rows][cols], A fp32 [tokens][lda], C fp32 [tokens][ldc];
+ * bias / mul (bf16 [rows]) nullable; accumulate != 0 adds into C (the residual update of a layer).  ops32 != 0 keeps the operands
+ * of the matrix-core product in fp32 (v_mfma_f32_32x32x2_f32) instead of rounding them to bfloat16; up to 8 tokens the product is
+ * a weight-streaming fp32 dot either way.  fp32 accumulation, no atomics: deterministic. */
+int ifa_linear_bf16w(const void *w_bf16, size_t rows, size_t cols, const void *a_f32, size_t lda, size_t tokens, const void *bias_bf16,
+                     const void *mul_bf16, float alpha, int accumulate, int ops32, void *c_f32, size_t ldc, ifa_stream stream);
+/* x[t] = embed[token_t] + pe(pos_t), pe[2i] = sin(p base^(-2i/width)), pe[2i+1] = cos(same); angles formed in double */
+int ifa_embed_sinpos_f32(const void *embed_bf16, int vocab, int width, const int *tokens_dev, const int *positions_dev, size_t tokens,
+                         float base, void *x_f32, ifa_stream stream);
+/* kind 0: RMS norm x / sqrt(mean(x^2) + eps) * w; kind 1: layer norm without bias (x - mean) / sqrt(var + eps) * w; w bf16 nullable */
+int ifa_layernorm_f32(int kind, const void *x_f32, size_t ldx, size_t rows, size_t cols, const void *w_bf16, float eps, void *y_f32, size_t ldy,
+                      ifa_stream stream);
+/* out[t][c] = act(gu[t][c]) * gu[t][cols + c]; kind 0 silu, 1 gelu (tanh form), 2 relu */
+int ifa_glu_f32(int kind, const void *gate_up_f32, size_t ld, size_t rows, size_t cols, void *out_f32, size_t ldo, ifa_stream stream);
+/* greedy argmax per row (lowest index on ties); excluded_dev = {count <= 3, id, id, id} nullable */
+int ifa_argmax_rows_f32(const void *logits_f32, size_t n, size_t row_stride, size_t rows, const int *excluded_dev, int *out_dev, ifa_stream stream);
+int ifa_convert_f32_f16(const void *src_f32, size_t n, void *dst_f16, ifa_stream stream);
+
+/* A step's rows are described by sequences: rows [row0, row0 + n) are positions [pos0, pos0 + n) of the sequence whose cache and
+ * state live in slot `slot`; row_seq_dev[row] = index of the row's sequence.  slot_base_dev[slot] = base pointer (fp32) of the
+ * slot's arena; *_off = offset in floats of a layer's part.  A sequence at pos0 == 0 starts from zero state whatever the slot holds. */
+typedef struct { int row0, n, pos0, slot; } ifa_seq_desc;
+/* short causal convolution per channel (w bf16 [channels][taps], last tap = current token) + SiLU; the last taps - 1 inputs of a
+ * sequence are carried in its slot ([taps - 1][channels]; ifa_shortconv_tail_f32 advances them AFTER the step's rows are computed).
+ * Then channels [0, norm_cols) become unit vectors in groups of group_dim (x / sqrt(sum x^2 + l2_eps)) and channels [0, scale_cols)
+ * are multiplied by scale. */
+int ifa_shortconv_silu_f32(const void *x_f32, size_t ldx, int channels, int taps, const void *w_bf16, const void *seqs_dev, const int *row_seq_dev,
+                           size_t rows, void *const *slot_base_dev, size_t state_off, int norm_cols, int group_dim, float l2_eps, int scale_cols,
+                           float scale, void *y_f32, size_t ldy, ifa_stream stream);
+int ifa_shortconv_tail_f32(const void *x_f32, size_t ldx, int channels, int taps, const void *seqs_dev, int n_seqs, void *const *slot_base_dev,
+                           size_t state_off, ifa_stream stream);
+/* gates of the gated delta rule: beta = sigmoid(b), decay = exp(-exp(A_log[h]) * softplus(a + dt_bias[h])); outputs fp32 [rows][heads] */
+int ifa_delta_gates_f32(const void *b_f32, size_t ldb, const void *a_f32, size_t lda, int heads, size_t rows, const void *a_log_bf16,
+                        const void *dt_bias_bf16, void *beta_f32, void *decay_f32, ifa_stream stream);
+/* per-head matrix state S [dk][dv] (fp32, in the slot: [heads][dk][dv]) advanced token by token;
+ * kind 0: S <- d_h S + k v^T, o = S^T q (decay_head_f32 [heads]); kind 1 (gated delta rule): S <- g S; u = beta (v - S^T k);
+ * S <- S + k u^T; o = S^T q (decay_row / beta_row fp32 [rows][heads]).  Head h reads q / k head h / (heads / qk_heads).
+ * in_act != 0: q, k, v pass SiLU as they are read.  dk <= 256. */
+int ifa_state_scan_f32(int kind, int in_act, const void *q_f32, size_t ldq, const void *k_f32, size_t ldk, const void *v_f32, size_t ldv, int heads,
+                       int qk_heads, int dk, int dv, const void *decay_head_f32, const void *decay_row_f32, const void *beta_row_f32,
+                       const void *seqs_dev, int n_seqs, void *const *slot_base_dev, size_t state_off, void *out_f32, size_t ldo, ifa_stream stream);
+/* y = o / sqrt(mean_group(o^2) + eps) * w[c % wlen] * act(gate); gate_act 0 sigmoid, 1 silu; groups of `group` channels; y may be o */
+int ifa_gated_groupnorm_f32(const void *o_f32, size_t ldo, size_t rows, int channels, int group, const void *w_bf16, int wlen, const void *gate_f32,
+                            size_t ldg, int gate_act, float eps, void *y_f32, size_t ldy, ifa_stream stream);
+/* rows of a step into the fp32 K / V cache of their sequences ([max_ctx][kv_heads * dim] each): K = k / rms_head(k) if norm_k, V = v */
+int ifa_kv_store_f32(const void *k_f32, size_t ldk, const void *v_f32, size_t ldv, int kv_heads, int dim, int norm_k, float eps, const void *seqs_dev,
+                     const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t k_off, size_t v_off, ifa_stream stream);
+/* softmax attention of the step's rows over their sequences' caches: query i sees key j iff j <= i and (i - j < window or
+ * j < keep_first); q RMS-normed per head if norm_q; score = q.k * scale, soft cap cap * tanh(score / cap) if softcap > 0, + bias
+ * rel[bucket_of[i - j]][head] if rel (bf16 [n_buckets][heads], bucket_of_dev: int per distance 0 .. max_ctx - 1); sink_bf16 [heads]
+ * (nullable): exp(sink) joins the denominator.  dim <= 256.  out fp32 [rows][heads * dim]. */
+int ifa_attention_window_f32(const void *q_f32, size_t ldq, int heads, int kv_heads, int dim, int norm_q, float eps, float scale, float softcap,
+                             int window, int keep_first, const void *rel_bf16, const int *bucket_of_dev, int n_buckets, const void *sink_bf16,
+                             const void *seqs_dev, const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t k_off, size_t v_off,
+                             void *out_f32, size_t ldo, ifa_stream stream);
+
+/* ======================================================================== */
+/* Layer-list worker: a decoder whose layers are given one by one, each with its own sequence mixer, a 32-bit residual       */
+/* stream and bfloat16 weights (csrc/ifa_engine_layered.hip).  It is an ifa_model: finalize / kv_slots / select_kv /        */
+/* forward / decode / decode_batch / set_option / set_excluded_tokens / get_buffer / destroy work as above (a "KV slot" holds */
+/* the key / value rows AND the recurrent states of one query); the tensor-parallel entry points decline.                   */
+/* A layer: h = norm1(x); x <- x + ls1 * mixer(h) + ls2 * ffn(h)  (one norm, both sub-layers read it).                      */
+/* ======================================================================== */
+enum { IFA_MIX_WINDOW_LINEAR = 1,   /* windowed softmax attention (values = keys as projected) + decayed linear attention, side by side */
+       IFA_MIX_GATED_DELTA = 2 };   /* gated delta rule behind short convolutions */
+typedef struct {
+    int mixer;                       /* IFA_MIX_* */
+    int ffn;                         /* width of the gated feed-forward (GELU tanh, biases); 0 = none */
+    /* windowed attention */
+    int a_heads, a_kv_heads, a_dim, a_window, a_keep_first, a_buckets, a_bias_max;
+    float a_scale, a_softcap, a_out_scale;
+    /* decayed linear attention (decays: tensor IFA_LT_L_DECAY) */
+    int l_heads, l_dim, l_vdim;
+    float l_out_scale;
+    /* gated delta rule */
+    int d_heads, d_kv_heads, d_dim, d_vdim, d_conv;
+} ifa_layer_spec;
+typedef struct {
+    int width, vocab, max_ctx, n_layers, device;
+    int ops32;                       /* 1: matrix products keep fp32 operands (exact mode); 0: operands rounded to bfloat16 */
+    float eps, pos_base;             /* eps of every norm of the stack; base of the sinusoidal position vector (10000) */
+} ifa_layered_config;
+/* tensors of a layer-list model (global ones use IFA_T_EMBD / IFA_T_OUT_NORM / IFA_T_LM_HEAD with layer = -1) */
+enum {
+    IFA_LT_NORM1 = 40, IFA_LT_LS1, IFA_LT_LS2, IFA_LT_FFN_GATE, IFA_LT_FFN_GATE_B, IFA_LT_FFN_UP, IFA_LT_FFN_UP_B, IFA_LT_FFN_DOWN, IFA_LT_FFN_DOWN_B,
+    IFA_LT_A_Q, IFA_LT_A_K, IFA_LT_A_REL, IFA_LT_A_SINK, IFA_LT_A_O,
+    IFA_LT_L_Q, IFA_LT_L_K, IFA_LT_L_V, IFA_LT_L_G, IFA_LT_L_O, IFA_LT_L_NORM, IFA_LT_L_DECAY /* fp32 [heads] */,
+    IFA_LT_D_Q, IFA_LT_D_K, IFA_LT_D_V, IFA_LT_D_QCONV, IFA_LT_D_KCONV, IFA_LT_D_VCONV, IFA_LT_D_B, IFA_LT_D_A, IFA_LT_D_ALOG, IFA_LT_D_DTBIAS,
+    IFA_LT_D_G, IFA_LT_D_NORM, IFA_LT_D_O, IFA_LT_END
+};
+int ifa_model_create_layered(const ifa_layered_config *cfg, const ifa_layer_spec *layers, ifa_model **out);
+/* a tensor from HOST memory: dtype IFA_BF16 (bit patterns) or IFA_F32 (IFA_LT_L_DECAY only); shapes are checked against the specs */
+int ifa_model_set_tensor_host(ifa_model *m, int layer, int tensor_id, int dtype, const void *host_src, size_t rows, size_t cols);
+/* fp32 logits of the most recent forward / decode_batch step (device pointer; rows x cols); the F16 logits_out of those calls
+ * is a rounded copy of these */
+int ifa_model_logits_f32(ifa_model *m, void **dptr, size_t *rows, size_t *cols);
+/* One step over several queries at once, prompts and single tokens mixed: query q brings seq_lens[q] tokens (all queries' tokens
+ * concatenated in tokens_host) at positions [seq_pos0[q], ...) on its slot seq_slots[q] (distinct).  all_logits 0: the fp32 logits
+ * (ifa_model_logits_f32) hold one row per query, that of its last token; 1: one row per token, in order.  next_tokens_host[q]:
+ * greedy token after query q's last row.  A row's result does not depend on what else is in the step. */
+int ifa_model_step_seqs(ifa_model *m, int n_seqs, const int *tokens_host, const int *seq_lens, const int *seq_pos0, const int *seq_slots, int all_logits,
+                        int *next_tokens_host);
+/* 1 for a layer-list model, 0 for the standard network */
+int ifa_model_is_layered(const ifa_model *m);
 
 #ifdef __cplusplus
 }

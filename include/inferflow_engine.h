@@ -18,6 +18,11 @@ typedef struct ifa_engine ifa_engine;
 
 /* InferenceEngine::LoadConfig(config_path, section, data_root_dir) + Init(); NULL on failure */
 ifa_engine *ifa_engine_create(const char *ini_path, const char *section, const char *data_root_dir);
+/* an engine for a bare model directory whose config.json names a registered layer-list architecture (+ model.safetensors), no .ini:
+ * compute_dtype "bfloat16" | "float32" (NULL = bfloat16), max_context_len tokens per query, max_concurrent_queries slots;
+ * return_output_tensors != 0: every step keeps its fp32 logits for ifa_engine_last_logits_f32.  NULL on failure */
+ifa_engine *ifa_engine_create_from_dir(const char *model_dir, const char *compute_dtype, int max_context_len, int max_concurrent_queries,
+                                       int return_output_tensors);
 void ifa_engine_destroy(ifa_engine *e);
 const char *ifa_engine_last_error(void);
 
@@ -54,6 +59,9 @@ int ifa_engine_infer(ifa_engine *e, int *query_ids, int *next_tokens, int capaci
 int ifa_engine_commit(ifa_engine *e, const int *query_ids, const int *tokens, const int *is_end, int n);
 /* rows/cols of the logits kept from the last Infer() for this query; copies min(capacity, rows*cols) halfs */
 int ifa_engine_last_logits(ifa_engine *e, int query_id, uint16_t *dst_f16, size_t capacity, int *rows, int *cols);
+
+/* the same in 32-bit floats (return_output_tensors_f32; layer-list models) */
+int ifa_engine_last_logits_f32(ifa_engine *e, int query_id, float *dst_f32, size_t capacity, int *rows, int *cols);
 
 /* InferenceResult::perf_stat of the last Infer() (InferencePerfStat::time_map, src/transformer/inference_types.h): up to `capacity`
  * (key, milliseconds) pairs in ascending key order; returns how many keys there are.  Key 0 = the step end to end

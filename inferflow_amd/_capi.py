@@ -148,6 +148,24 @@ SIGNATURES = {
     "ifa_model_tp_prefill": (_i, [_vp, _vp, _vp, _i, _i, _vp, _vp]),
     "ifa_model_tp_decode_batch": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp]),
     "ifa_model_get_tensor": (_i, [_vp, _i, _i, _vp, C.POINTER(_vp), C.POINTER(_sz), C.POINTER(_sz)]),
+    "ifa_linear_bf16w": (_i, [_vp, _sz, _sz, _vp, _sz, _sz, _vp, _vp, _f, _i, _i, _vp, _sz, _vp]),
+    "ifa_embed_sinpos_f32": (_i, [_vp, _i, _i, _vp, _vp, _sz, _f, _vp, _vp]),
+    "ifa_layernorm_f32": (_i, [_i, _vp, _sz, _sz, _sz, _vp, _f, _vp, _sz, _vp]),
+    "ifa_glu_f32": (_i, [_i, _vp, _sz, _sz, _sz, _vp, _sz, _vp]),
+    "ifa_argmax_rows_f32": (_i, [_vp, _sz, _sz, _sz, _vp, _vp, _vp]),
+    "ifa_convert_f32_f16": (_i, [_vp, _sz, _vp, _vp]),
+    "ifa_shortconv_silu_f32": (_i, [_vp, _sz, _i, _i, _vp, _vp, _vp, _sz, _vp, _sz, _i, _i, _f, _i, _f, _vp, _sz, _vp]),
+    "ifa_shortconv_tail_f32": (_i, [_vp, _sz, _i, _i, _vp, _i, _vp, _sz, _vp]),
+    "ifa_delta_gates_f32": (_i, [_vp, _sz, _vp, _sz, _i, _sz, _vp, _vp, _vp, _vp, _vp]),
+    "ifa_state_scan_f32": (_i, [_i, _i, _vp, _sz, _vp, _sz, _vp, _sz, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _sz, _vp, _sz, _vp]),
+    "ifa_gated_groupnorm_f32": (_i, [_vp, _sz, _sz, _i, _i, _vp, _i, _vp, _sz, _i, _f, _vp, _sz, _vp]),
+    "ifa_kv_store_f32": (_i, [_vp, _sz, _vp, _sz, _i, _i, _i, _f, _vp, _vp, _sz, _vp, _sz, _sz, _vp]),
+    "ifa_attention_window_f32": (_i, [_vp, _sz, _i, _i, _i, _i, _f, _f, _f, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _sz, _vp, _sz, _sz, _vp, _sz, _vp]),
+    "ifa_model_create_layered": (_i, [_vp, _vp, C.POINTER(_vp)]),
+    "ifa_model_set_tensor_host": (_i, [_vp, _i, _i, _i, _vp, _sz, _sz]),
+    "ifa_model_logits_f32": (_i, [_vp, C.POINTER(_vp), C.POINTER(_sz), C.POINTER(_sz)]),
+    "ifa_model_step_seqs": (_i, [_vp, _i, _vp, _vp, _vp, _vp, _i, _vp]),
+    "ifa_model_is_layered": (_i, [_vp]),
     "ifa_model_get_expert_tensor": (_i, [_vp, _i, _i, _i, _vp, C.POINTER(_vp), C.POINTER(_sz), C.POINTER(_sz)]),
 }
 
@@ -157,6 +175,8 @@ _ip = C.POINTER(C.c_int)
 ENGINE_SIGNATURES = {
     "ifa_engine_create": (_vp, [C.c_char_p, C.c_char_p, C.c_char_p]),
     "ifa_engine_destroy": (None, [_vp]),
+    "ifa_engine_create_from_dir": (_vp, [C.c_char_p, C.c_char_p, _i, _i, _i]),
+    "ifa_engine_last_logits_f32": (_i, [_vp, _i, _vp, _sz, _ip, _ip]),
     "ifa_engine_last_error": (C.c_char_p, []),
     "ifa_engine_add_query": (_i, [_vp, _ip, _i]),
     "ifa_engine_add_query_ex": (_i, [_vp, _ip, _i, _i, _i, _f]),

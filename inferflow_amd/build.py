@@ -19,6 +19,8 @@ HIPCC_FLAGS = [
     "--offload-arch=" + ARCH, "-O3", "-std=c++17", "-fPIC",
     # exact-rounding parity with the host-compiled reference codecs
     "-ffp-contract=off",
+    # no packed fp32 instructions (v_pk_add / mul / fma_f32) from ordinary float code
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     # leading scalar kernel arguments arrive in SGPRs at wave launch (gfx940+), see k_dec_gemv
     "-mllvm", "-amdgpu-kernarg-preload-count=8",
     "-Wall", "-Wno-unused-function", "-Wno-unused-variable", "-Wno-unused-but-set-variable",
@@ -152,6 +154,8 @@ def build_library(force=False, verbose=False, jobs=None):
                            os.path.join(BIN_DIR, "ifa_perplexity"), "-L", LIB_DIR, "-linferflow_amd", "-Wl,-rpath,$ORIGIN/../lib"])
     subprocess.check_call([cxx] + HOST_FLAGS + ["-I", inc, "-I", HOST, os.path.join(HOST, "inferflow_service_main.cc"), "-o",
                            os.path.join(BIN_DIR, "ifa_service"), "-L", LIB_DIR, "-linferflow_amd", "-Wl,-rpath,$ORIGIN/../lib"])
+    subprocess.check_call([cxx] + HOST_FLAGS + ["-I", inc, "-I", HOST, os.path.join(HOST, "trace_run_main.cc"), "-o",
+                           os.path.join(BIN_DIR, "ifa_trace_run"), "-L", LIB_DIR, "-linferflow_amd", "-Wl,-rpath,$ORIGIN/../lib"])
     return LIB_PATH
 
 

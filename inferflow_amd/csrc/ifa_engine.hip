@@ -276,6 +276,7 @@ int ifa_model_create(const ifa_model_config *cfg, ifa_model **out)
 int ifa_model_destroy(ifa_model *m)
 {
     if (!m) return IFA_OK;
+    if (m->vt) return m->vt->destroy(m);
     (void)hipSetDevice(m->cfg.device);
     if (m->stream) (void)hipStreamSynchronize(m->stream);
     drop_graphs(m);
@@ -339,6 +340,7 @@ int ifa_model_set_tensor(ifa_model *m, int layer, int tensor_id, int expert, int
                          size_t rows, size_t cols)
 {
     IFA_REQUIRE(m && dev_src, "ifa_model_set_tensor: null pointer");
+    IFA_STD_ONLY(m, "ifa_model_set_tensor");
     IFA_REQUIRE(tensor_id >= 0 && tensor_id < T_MAX, "ifa_model_set_tensor: tensor id %d", tensor_id);
     IFA_REQUIRE(expert < 0 || (expert < m->cfg.experts && layer >= 0 && (tensor_id == T_W1 || tensor_id == T_W2 || tensor_id == T_W3)),
                 "ifa_model_set_tensor: expert %d (of %d) / tensor %d", expert, m->cfg.experts, tensor_id);
@@ -429,6 +431,7 @@ int ifa_model_set_tensor_f16(ifa_model *m, int layer, int tensor_id, int expert,
 int ifa_model_finalize(ifa_model *m)
 {
     IFA_REQUIRE(m, "ifa_model_finalize: null model");
+    if (m->vt) return m->vt->finalize(m);
     IFA_HIP_CHECK(hipSetDevice(m->cfg.device));
     (void)wait_err_word();       // (the device's wait-error word exists before any step can be captured: ifa_host.h)
     const ifa_model_config &c = m->cfg;
@@ -479,6 +482,7 @@ int ifa_model_finalize(ifa_model *m)
 
 int ifa_model_reset(ifa_model *m)
 {
+    if (m && m->vt) return m->vt->reset(m);
     IFA_REQUIRE(m && m->finalized, "ifa_model_reset: model not finalized");
     IFA_HIP_CHECK(hipSetDevice(m->cfg.device));
     for (Layer &L : m->layers) {
@@ -491,6 +495,7 @@ int ifa_model_reset(ifa_model *m)
 
 int ifa_model_kv_slots(ifa_model *m, int n_slots)
 {
+    if (m && m->vt) return m->vt->kv_slots(m, n_slots);
     IFA_REQUIRE(m && m->finalized, "ifa_model_kv_slots: model not finalized");
     IFA_REQUIRE(n_slots >= 1 && n_slots <= 4096, "ifa_model_kv_slots: n_slots %d", n_slots);
     IFA_HIP_CHECK(hipSetDevice(m->cfg.device));
@@ -515,6 +520,7 @@ int ifa_model_kv_slots(ifa_model *m, int n_slots)
 
 int ifa_model_select_kv(ifa_model *m, int slot)
 {
+    if (m && m->vt) return m->vt->select_kv(m, slot);
     IFA_REQUIRE(m && m->finalized, "ifa_model_select_kv: model not finalized");
     if (m->slots.empty()) m->slots.resize(1);
     IFA_REQUIRE(slot >= 0 && slot < (int)m->slots.size(), "ifa_model_select_kv: slot %d of %zu", slot, m->slots.size());
@@ -538,6 +544,7 @@ int ifa_model_select_kv(ifa_model *m, int slot)
 int ifa_model_set_option(ifa_model *m, const char *name, int value)
 {
     IFA_REQUIRE(m && name, "ifa_model_set_option: null pointer");
+    if (m->vt) return m->vt->set_option(m, name, value);
     struct { const char *n; int *p; } opts[] = {
         {"fused", &m->opt_fused}, {"graph", &m->opt_graph}, {"rpw_qkv", &m->opt_rpw_qkv}, {"rpw_wo", &m->opt_rpw_wo},
         {"rpw_ffn", &m->opt_rpw_ffn}, {"rpw_w2", &m->opt_rpw_w2}, {"rpw_lm", &m->opt_rpw_lm}, {"trace", &m->opt_trace},
@@ -560,6 +567,7 @@ int ifa_model_set_option(ifa_model *m, const char *name, int value)
 int ifa_model_perf_stat(ifa_model *m, int *keys_out, float *ms_out, int cap, int *n_out, int clear)
 {
     IFA_REQUIRE(m && n_out && cap >= 0 && (cap == 0 || (keys_out && ms_out)), "ifa_model_perf_stat: null pointer");
+    IFA_STD_ONLY(m, "ifa_model_perf_stat");
     IFA_HIP_CHECK(hipSetDevice(m->cfg.device));
     int rc = perf_collect(m);
     if (rc) return rc;
@@ -575,6 +583,7 @@ int ifa_model_perf_stat(ifa_model *m, int *keys_out, float *ms_out, int cap, int
 
 int ifa_model_set_excluded_tokens(ifa_model *m, const int *ids_host, int n)
 {
+    if (m && m->vt) return m->vt->set_excluded_tokens(m, ids_host, n);
     IFA_REQUIRE(m && m->finalized, "ifa_model_set_excluded_tokens: model not finalized");
     IFA_REQUIRE(n >= 0 && n <= 3 && (n == 0 || ids_host), "ifa_model_set_excluded_tokens: n %d (0..3)", n);
     int v[4] = {n, -1, -1, -1};
@@ -587,6 +596,7 @@ int ifa_model_set_excluded_tokens(ifa_model *m, const int *ids_host, int n)
 int ifa_model_fused_supported(ifa_model *m, char *why, size_t why_len)
 {
     IFA_REQUIRE(m, "ifa_model_fused_supported: null model");
+    if (m->vt) { if (why && why_len) { strncpy(why, "layer-list model", why_len - 1); why[why_len - 1] = 0; } return 0; }
     std::string w;
     bool ok = fused_supported(m, &w);
     if (why && why_len) { strncpy(why, w.c_str(), why_len - 1); why[why_len - 1] = 0; }
@@ -596,6 +606,7 @@ int ifa_model_fused_supported(ifa_model *m, char *why, size_t why_len)
 int ifa_model_get_buffer(ifa_model *m, const char *name, int layer, void **dptr, size_t *bytes)
 {
     IFA_REQUIRE(m && name && dptr, "ifa_model_get_buffer: null pointer");
+    if (m->vt) return m->vt->get_buffer(m, name, layer, dptr, bytes);
     const ifa_model_config &c = m->cfg;
     size_t b = 0; void *p = nullptr;
     if (!strcmp(name, "logits")) { p = m->logits; b = (size_t)c.vocab * 2; }
@@ -624,6 +635,7 @@ void *ifa_model_stream(ifa_model *m) { return m ? (void *)m->stream : nullptr; }
 int ifa_model_set_stream(ifa_model *m, ifa_stream stream)
 {
     IFA_REQUIRE(m, "ifa_model_set_stream: null model");
+    IFA_STD_ONLY(m, "ifa_model_set_stream");
     IFA_HIP_CHECK(hipSetDevice(m->cfg.device));
     if (m->stream) IFA_HIP_CHECK(hipStreamSynchronize(m->stream));
     if (m->stream) (void)ifa_gemm_release_stream((ifa_stream)m->stream);
@@ -637,6 +649,7 @@ int ifa_model_set_stream(ifa_model *m, ifa_stream stream)
 int ifa_model_get_tensor(ifa_model *m, int layer, int tensor_id, int *dtype, void **dptr, size_t *rows, size_t *cols)
 {
     IFA_REQUIRE(m && tensor_id >= 0 && tensor_id < T_MAX, "ifa_model_get_tensor: bad arguments");
+    IFA_STD_ONLY(m, "ifa_model_get_tensor");
     const Tensor *t;
     if (tensor_id < 10) t = &m->g[tensor_id];
     else {
@@ -653,6 +666,7 @@ int ifa_model_get_tensor(ifa_model *m, int layer, int tensor_id, int *dtype, voi
 // W1 / W2 / W3 of one expert of a mixture-of-experts layer (the layer's own tensor ids name the dense FFN)
 int ifa_model_get_expert_tensor(ifa_model *m, int layer, int expert, int tensor_id, int *dtype, void **dptr, size_t *rows, size_t *cols)
 {
+    IFA_STD_ONLY(m, "ifa_model_get_expert_tensor");
     IFA_REQUIRE(m && layer >= 0 && layer < m->cfg.layers, "ifa_model_get_expert_tensor: layer %d", layer);
     IFA_REQUIRE(tensor_id == T_W1 || tensor_id == T_W2 || tensor_id == T_W3, "ifa_model_get_expert_tensor: tensor id %d (w1 / w2 / w3 only)", tensor_id);
     const Layer &L = m->layers[(size_t)layer];

@@ -115,6 +115,7 @@ bool has_post_norms(const ifa_model *m)
 // Can the fused decode path run this model?  (otherwise decode falls back to forward())
 bool fused_supported(const ifa_model *m, std::string *why)
 {
+    if (m->vt) { if (why) *why = "layer-list model"; return false; }
     const ifa_model_config &c = m->cfg;
     auto fail = [&](const char *s) { if (why) *why = s; return false; };
     if (has_post_norms(m)) return fail("post norms (self_attn.post_norm / feed_forward.post_norm) use the op-by-op path");
@@ -721,6 +722,7 @@ extern "C" {
 
 int ifa_model_decode(ifa_model *m, int first_token, int start_pos, int n_steps, int *out_tokens_host, float *elapsed_ms)
 {
+    if (m && m->vt) return m->vt->decode(m, first_token, start_pos, n_steps, out_tokens_host, elapsed_ms, false);
     return decode_impl(m, first_token, start_pos, n_steps, out_tokens_host, elapsed_ms, false);
 }
 
@@ -730,6 +732,7 @@ int ifa_model_decode(ifa_model *m, int first_token, int start_pos, int n_steps, 
 // touched (the token / position words are rewritten by every call anyway).
 int ifa_model_decode_prepare(ifa_model *m, int start_pos, int n_steps)
 {
+    if (m && m->vt) return m->vt->decode(m, 0, start_pos, n_steps, nullptr, nullptr, true);
     return decode_impl(m, 0, start_pos, n_steps, nullptr, nullptr, true);
 }
 
@@ -865,6 +868,7 @@ extern "C" {
 
 int ifa_model_time_kernel(ifa_model *m, int which, int iters, float *avg_us)
 {
+    IFA_STD_ONLY(m, "ifa_model_time_kernel");
     IFA_REQUIRE(m && m->finalized && avg_us, "ifa_model_time_kernel: bad arguments");
     IFA_REQUIRE(iters > 0 && which >= 0 && which <= 9, "ifa_model_time_kernel: which %d iters %d", which, iters);
     IFA_HIP_CHECK(hipSetDevice(m->cfg.device));

@@ -741,6 +741,7 @@ int ifa_model_forward(ifa_model *m, const int *tokens_host, int n_tokens, int pr
                       int *next_token_host)
 {
     IFA_REQUIRE(m && m->finalized, "ifa_model_forward: model not finalized");
+    if (m->vt) return m->vt->forward(m, tokens_host, n_tokens, prefix_len, logits_out_dev, next_token_host);
     IFA_REQUIRE(tokens_host, "ifa_model_forward: null tokens");
     IFA_HIP_CHECK(hipSetDevice(m->cfg.device));
     if (m->opt_exact_order) {      // order-exact: the tokens one by one through the single-row step (the reference's T = 1 branch for every row)
@@ -772,6 +773,7 @@ int ifa_model_decode_batch(ifa_model *m, int n, const int *tokens_host, const in
                            int *next_tokens_host, void *logits_out_dev)
 {
     IFA_REQUIRE(m && m->finalized, "ifa_model_decode_batch: model not finalized");
+    if (m->vt) return m->vt->decode_batch(m, n, tokens_host, positions_host, kv_slots_host, next_tokens_host, logits_out_dev);
     IFA_REQUIRE(n >= 1 && n <= ifa_model::RING && tokens_host && positions_host && kv_slots_host, "ifa_model_decode_batch: bad arguments");
     IFA_HIP_CHECK(hipSetDevice(m->cfg.device));
     if (m->opt_exact_order) {      // order-exact: every query's row through the single-row step on ITS cache set (a batched step of the

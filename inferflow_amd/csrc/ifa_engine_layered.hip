@@ -1,0 +1,694 @@
+// ifa_engine_layered.hip -- the layer-list worker: a decoder given layer by layer, each layer with its own sequence mixer
+// (windowed softmax attention beside decayed linear attention, or the gated delta rule), one norm feeding mixer and
+// feed-forward in parallel, layer scales, a 32-bit residual stream and bfloat16 weights.  It answers the same ifa_model_*
+// entry points as the standard network (ifa_model_vtbl) so that the engine above drives both alike.
+//
+// Slots: what the standard network calls a KV slot holds, per query, ALL per-sequence memory of the stack in one arena:
+//   windowed attention   K rows (normed keys) and V rows [max_ctx][kv_heads * dim] fp32, addressed by position
+//   linear attention     S [heads][dk][dv] fp32
+//   gated delta rule     S [heads][dk][dv] fp32 + the last conv - 1 inputs of the short convolutions
+// An arena is allocated when its slot is first used; a sequence that starts at position 0 ignores what the slot held.
+//
+// A step = a list of sequences (ifa_seq_desc): forward() is one sequence of n tokens from position prefix_len,
+// decode_batch() n sequences of one token, decode() one sequence advanced token by token with the argmax fed back
+// on the device (the step's tables live in device memory, so the captured step replays for every token).
+// Per layer: norm1 -> ONE product for every projection that reads it (mixer inputs, gates, FFN gate | up; biases in the
+// epilogue) -> mixer kernels -> output products that add into the fp32 residual with layer scale and branch scale
+// in their epilogue -> GELU-gated FFN the same way.
+#include <algorithm>
+#include <cmath>
+#include <cstring>
+#include <string>
+#include <vector>
+#include "ifa_engine_state.h"
+#include "ifa_f32_common.h"
+
+using ifa32::bf16_t;
+
+namespace {
+
+struct LTensor { void *data = nullptr; int dtype = -1; size_t rows = 0, cols = 0; bool present() const { return data != nullptr; } };
+
+struct LLayer {
+    ifa_layer_spec spec;
+    LTensor t[IFA_LT_END - IFA_LT_NORM1];
+    // fused input projection: rows of every matrix that reads norm1's output, and its bias vector
+    bf16_t *w_in = nullptr, *b_in = nullptr; size_t n_in = 0;
+    size_t c_aq = 0, c_ak = 0, c_lq = 0, c_lk = 0, c_lv = 0, c_lg = 0, c_dq = 0, c_db = 0, c_da = 0, c_dg = 0, c_fg = 0;   // column offsets in the product
+    bf16_t *w_conv = nullptr; int conv_ch = 0;       // [q | k | v channels][taps]
+    int *bucket_of = nullptr;                         // distance -> bias row
+    // arena offsets (floats)
+    size_t o_k = 0, o_v = 0, o_lin = 0, o_rec = 0, o_conv = 0;
+    LTensor &T(int id) { return t[id - IFA_LT_NORM1]; }
+    const LTensor &T(int id) const { return t[id - IFA_LT_NORM1]; }
+};
+
+constexpr int MAX_SLOTS = 4096;
+
+} // namespace
+
+struct LayeredNet {
+    ifa_layered_config cfg;
+    std::vector<LLayer> layers;
+    LTensor embd, out_norm, lm_head;
+    size_t arena_floats = 0;
+    std::vector<float *> slot_ptr;       // host copy of the table (null: not allocated yet)
+    float **slot_base_dev = nullptr;
+    int n_slots = 1, cur_slot = 0;
+    // step tables: pinned staging + device
+    int *tab_pin = nullptr, *tab_dev = nullptr; size_t tab_rows = 0, tab_seqs = 0;
+    int *tokens_dev = nullptr, *pos_dev = nullptr, *row_seq_dev = nullptr; ifa_seq_desc *seqs_dev = nullptr;
+    int *excl_dev = nullptr, *next_dev = nullptr, *ring_dev = nullptr;
+    // activations (fp32), sized for scratch_rows
+    size_t scratch_rows = 0, n_in_max = 0, mix_max = 0, ffn_max = 0, heads_max = 0;
+    float *x = nullptr, *h = nullptr, *proj = nullptr, *m1 = nullptr, *m2 = nullptr, *m3 = nullptr, *beta = nullptr, *decay = nullptr, *logits = nullptr;
+    size_t logits_rows = 0, logits_cap = 0;
+    float *taps = nullptr; size_t taps_rows = 0; int opt_tap_layers = 0;
+    int opt_graph = 1;
+    hipGraphExec_t step_exec = nullptr; hipGraph_t step_graph = nullptr; int step_slot = -1;
+};
+
+namespace {
+
+int lay_free(void *p) { if (p) (void)hipFree(p); return 0; }
+
+void drop_step_graph(LayeredNet *n)
+{
+    if (n->step_exec) { (void)hipGraphExecDestroy(n->step_exec); n->step_exec = nullptr; }
+    if (n->step_graph) { (void)hipGraphDestroy(n->step_graph); n->step_graph = nullptr; }
+    n->step_slot = -1;
+}
+
+// rows x cols a tensor of this layer must have; false: the tensor does not belong to the layer's mixer
+bool expected_shape(const LayeredNet *n, const ifa_layer_spec &s, int id, size_t &r, size_t &c, bool &vec)
+{
+    const size_t W = (size_t)n->cfg.width;
+    vec = false;
+    const bool par = s.mixer == IFA_MIX_WINDOW_LINEAR, del = s.mixer == IFA_MIX_GATED_DELTA;
+    switch (id) {
+    case IFA_LT_NORM1: case IFA_LT_LS1: r = 1; c = W; vec = true; return true;
+    case IFA_LT_LS2: case IFA_LT_FFN_DOWN_B: r = 1; c = W; vec = true; return s.ffn > 0;
+    case IFA_LT_FFN_GATE: case IFA_LT_FFN_UP: r = (size_t)s.ffn; c = W; return s.ffn > 0;
+    case IFA_LT_FFN_GATE_B: case IFA_LT_FFN_UP_B: r = 1; c = (size_t)s.ffn; vec = true; return s.ffn > 0;
+    case IFA_LT_FFN_DOWN: r = W; c = (size_t)s.ffn; return s.ffn > 0;
+    case IFA_LT_A_Q: r = (size_t)s.a_heads * s.a_dim; c = W; return par;
+    case IFA_LT_A_K: r = (size_t)s.a_kv_heads * s.a_dim; c = W; return par;
+    case IFA_LT_A_REL: r = (size_t)s.a_buckets; c = (size_t)s.a_heads; return par;
+    case IFA_LT_A_SINK: r = 1; c = (size_t)s.a_heads; vec = true; return par;
+    case IFA_LT_A_O: r = W; c = (size_t)s.a_heads * s.a_dim; return par;
+    case IFA_LT_L_Q: case IFA_LT_L_K: r = (size_t)s.l_heads * s.l_dim; c = W; return par;
+    case IFA_LT_L_V: case IFA_LT_L_G: r = (size_t)s.l_heads * s.l_vdim; c = W; return par;
+    case IFA_LT_L_O: r = W; c = (size_t)s.l_heads * s.l_vdim; return par;
+    case IFA_LT_L_NORM: r = 1; c = (size_t)s.l_heads * s.l_vdim; vec = true; return par;
+    case IFA_LT_L_DECAY: r = 1; c = (size_t)s.l_heads; vec = true; return par;
+    case IFA_LT_D_Q: case IFA_LT_D_K: r = (size_t)s.d_kv_heads * s.d_dim; c = W; return del;
+    case IFA_LT_D_V: case IFA_LT_D_G: r = (size_t)s.d_heads * s.d_vdim; c = W; return del;
+    case IFA_LT_D_QCONV: case IFA_LT_D_KCONV: r = (size_t)s.d_kv_heads * s.d_dim; c = (size_t)s.d_conv; return del;
+    case IFA_LT_D_VCONV: r = (size_t)s.d_heads * s.d_vdim; c = (size_t)s.d_conv; return del;
+    case IFA_LT_D_B: case IFA_LT_D_A: r = (size_t)s.d_heads; c = W; return del;
+    case IFA_LT_D_ALOG: case IFA_LT_D_DTBIAS: r = 1; c = (size_t)s.d_heads; vec = true; return del;
+    case IFA_LT_D_NORM: r = 1; c = (size_t)s.d_vdim; vec = true; return del;
+    case IFA_LT_D_O: r = W; c = (size_t)s.d_heads * s.d_vdim; return del;
+    default: return false;
+    }
+}
+
+size_t align4(size_t v) { return (v + 3) & ~(size_t)3; }
+
+// distance -> row of the bias table: n for n < B / 2, then logarithmic up to bias_max, the last row beyond (formed in double)
+void build_buckets(std::vector<int> &out, int max_ctx, int B, int Dmax)
+{
+    out.resize((size_t)max_ctx);
+    const int half = B / 2;
+    for (int d = 0; d < max_ctx; d++) {
+        int b;
+        if (d < half || half <= 0) b = std::min(d, B - 1);
+        else if (Dmax <= half) b = B - 1;
+        else {
+            const double f = std::log((double)d / (double)half) / std::log((double)Dmax / (double)half) * (double)(B - half);
+            b = std::min(B - 1, half + (int)std::floor(f));
+        }
+        out[(size_t)d] = b;
+    }
+}
+
+int ensure_slot(ifa_model *m, int slot)
+{
+    LayeredNet *n = m->lay;
+    IFA_REQUIRE(slot >= 0 && slot < n->n_slots, "layer-list worker: slot %d of %d", slot, n->n_slots);
+    if (n->slot_ptr[(size_t)slot]) return IFA_OK;
+    float *p = nullptr;
+    IFA_HIP_CHECK(hipMalloc((void **)&p, std::max<size_t>(n->arena_floats, 4) * 4));
+    n->slot_ptr[(size_t)slot] = p;
+    IFA_HIP_CHECK(hipMemcpyAsync(n->slot_base_dev + slot, &n->slot_ptr[(size_t)slot], sizeof(float *), hipMemcpyHostToDevice, m->stream));
+    IFA_HIP_CHECK(hipStreamSynchronize(m->stream));
+    return IFA_OK;
+}
+
+int ensure_rows(ifa_model *m, size_t T, size_t nseq)
+{
+    LayeredNet *n = m->lay;
+    if (T > n->tab_rows || nseq > n->tab_seqs) {
+        IFA_HIP_CHECK(hipStreamSynchronize(m->stream));
+        drop_step_graph(n);
+        if (n->tab_pin) (void)hipHostFree(n->tab_pin);
+        lay_free(n->tab_dev);
+        n->tab_pin = nullptr; n->tab_dev = nullptr;
+        const size_t R = std::max(T, n->tab_rows), S = std::max(nseq, n->tab_seqs);
+        const size_t ints = 3 * R + 4 * S;
+        IFA_HIP_CHECK(hipHostMalloc((void **)&n->tab_pin, ints * 4, hipHostMallocDefault));
+        IFA_HIP_CHECK(hipMalloc((void **)&n->tab_dev, ints * 4));
+        n->tab_rows = R; n->tab_seqs = S;
+        n->tokens_dev = n->tab_dev; n->pos_dev = n->tab_dev + R; n->row_seq_dev = n->tab_dev + 2 * R; n->seqs_dev = (ifa_seq_desc *)(n->tab_dev + 3 * R);
+    }
+    if (T > n->scratch_rows) {
+        IFA_HIP_CHECK(hipStreamSynchronize(m->stream));
+        drop_step_graph(n);
+        float **bufs[] = {&n->x, &n->h, &n->proj, &n->m1, &n->m2, &n->m3, &n->beta, &n->decay};
+        for (float **b : bufs) { lay_free(*b); *b = nullptr; }
+        const size_t W = (size_t)n->cfg.width;
+        const size_t sz[] = {W, W, n->n_in_max, n->mix_max, n->mix_max, std::max<size_t>(n->ffn_max, 4), std::max<size_t>(n->heads_max, 4), std::max<size_t>(n->heads_max, 4)};
+        for (size_t i = 0; i < 8; i++) IFA_HIP_CHECK(hipMalloc((void **)bufs[i], T * sz[i] * 4));
+        n->scratch_rows = T;
+    }
+    return IFA_OK;
+}
+
+int ensure_logits(ifa_model *m, size_t rows)
+{
+    LayeredNet *n = m->lay;
+    if (rows > n->logits_cap) {
+        IFA_HIP_CHECK(hipStreamSynchronize(m->stream));
+        drop_step_graph(n);
+        lay_free(n->logits); n->logits = nullptr;
+        IFA_HIP_CHECK(hipMalloc((void **)&n->logits, rows * (size_t)n->cfg.vocab * 4));
+        n->logits_cap = rows;
+    }
+    return IFA_OK;
+}
+
+int linear(ifa_model *m, const bf16_t *W, size_t N, size_t K, const float *A, size_t lda, size_t T, const bf16_t *bias, const bf16_t *mul, float alpha,
+           int accumulate, float *C, size_t ldc)
+{
+    return ifa_linear_bf16w(W, N, K, A, lda, T, bias, mul, alpha, accumulate, m->lay->cfg.ops32, C, ldc, (ifa_stream)m->stream);
+}
+
+// the layers of one step over T rows / nseq sequences whose tables are already on the device; leaves the residual in n->x
+int run_layers(ifa_model *m, size_t T, int nseq)
+{
+    LayeredNet *n = m->lay;
+    const ifa_layered_config &c = n->cfg;
+    const size_t W = (size_t)c.width;
+    ifa_stream s = (ifa_stream)m->stream;
+    void *const *slots = (void *const *)n->slot_base_dev;
+    int rc;
+    if ((rc = ifa_embed_sinpos_f32(n->embd.data, c.vocab, c.width, n->tokens_dev, n->pos_dev, T, c.pos_base, n->x, s))) return rc;
+    for (size_t li = 0; li < n->layers.size(); li++) {
+        LLayer &L = n->layers[li];
+        const ifa_layer_spec &sp = L.spec;
+        const bf16_t *ls1 = (const bf16_t *)L.T(IFA_LT_LS1).data;
+        if ((rc = ifa_layernorm_f32(1, n->x, W, T, W, L.T(IFA_LT_NORM1).data, c.eps, n->h, W, s))) return rc;
+        const size_t NI = L.n_in;
+        if ((rc = linear(m, L.w_in, NI, W, n->h, W, T, L.b_in, nullptr, 1.0f, 0, n->proj, NI))) return rc;
+        if (sp.mixer == IFA_MIX_WINDOW_LINEAR) {
+            const size_t AQ = (size_t)sp.a_heads * sp.a_dim, LV = (size_t)sp.l_heads * sp.l_vdim;
+            // windowed attention: the values are the keys as projected; the cache's K rows hold the normed keys
+            if ((rc = ifa_kv_store_f32(n->proj + L.c_ak, NI, n->proj + L.c_ak, NI, sp.a_kv_heads, sp.a_dim, 1, c.eps, n->seqs_dev, n->row_seq_dev, T, slots,
+                                       L.o_k, L.o_v, s))) return rc;
+            if ((rc = ifa_attention_window_f32(n->proj + L.c_aq, NI, sp.a_heads, sp.a_kv_heads, sp.a_dim, 1, c.eps, sp.a_scale, sp.a_softcap, sp.a_window,
+                                               sp.a_keep_first, L.T(IFA_LT_A_REL).data, L.bucket_of, sp.a_buckets, L.T(IFA_LT_A_SINK).data, n->seqs_dev,
+                                               n->row_seq_dev, T, slots, L.o_k, L.o_v, n->m1, AQ, s))) return rc;
+            if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_A_O).data, W, AQ, n->m1, AQ, T, nullptr, ls1, sp.a_out_scale, 1, n->x, W))) return rc;
+            // decayed linear attention
+            if ((rc = ifa_state_scan_f32(0, 1, n->proj + L.c_lq, NI, n->proj + L.c_lk, NI, n->proj + L.c_lv, NI, sp.l_heads, sp.l_heads, sp.l_dim, sp.l_vdim,
+                                         L.T(IFA_LT_L_DECAY).data, nullptr, nullptr, n->seqs_dev, nseq, slots, L.o_lin, n->m2, LV, s))) return rc;
+            if ((rc = ifa_gated_groupnorm_f32(n->m2, LV, T, (int)LV, (int)LV, L.T(IFA_LT_L_NORM).data, (int)LV, n->proj + L.c_lg, NI, 0, c.eps, n->m2, LV, s))) return rc;
+            if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_L_O).data, W, LV, n->m2, LV, T, nullptr, ls1, sp.l_out_scale, 1, n->x, W))) return rc;
+        } else {
+            const size_t QK = (size_t)sp.d_kv_heads * sp.d_dim, DV = (size_t)sp.d_heads * sp.d_vdim, C = (size_t)L.conv_ch;
+            if ((rc = ifa_shortconv_silu_f32(n->proj + L.c_dq, NI, (int)C, sp.d_conv, L.w_conv, n->seqs_dev, n->row_seq_dev, T, slots, L.o_conv, (int)(2 * QK),
+                                             sp.d_dim, 1e-6f, (int)QK, 1.0f / sqrtf((float)sp.d_dim), n->m1, C, s))) return rc;
+            if ((rc = ifa_shortconv_tail_f32(n->proj + L.c_dq, NI, (int)C, sp.d_conv, n->seqs_dev, nseq, slots, L.o_conv, s))) return rc;
+            if ((rc = ifa_delta_gates_f32(n->proj + L.c_db, NI, n->proj + L.c_da, NI, sp.d_heads, T, L.T(IFA_LT_D_ALOG).data, L.T(IFA_LT_D_DTBIAS).data,
+                                          n->beta, n->decay, s))) return rc;
+            if ((rc = ifa_state_scan_f32(1, 0, n->m1, C, n->m1 + QK, C, n->m1 + 2 * QK, C, sp.d_heads, sp.d_kv_heads, sp.d_dim, sp.d_vdim, nullptr, n->decay,
+                                         n->beta, n->seqs_dev, nseq, slots, L.o_rec, n->m2, DV, s))) return rc;
+            if ((rc = ifa_gated_groupnorm_f32(n->m2, DV, T, (int)DV, sp.d_vdim, L.T(IFA_LT_D_NORM).data, sp.d_vdim, n->proj + L.c_dg, NI, 1, c.eps, n->m2, DV, s))) return rc;
+            if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_D_O).data, W, DV, n->m2, DV, T, nullptr, ls1, 1.0f, 1, n->x, W))) return rc;
+        }
+        if (sp.ffn > 0) {
+            const size_t F = (size_t)sp.ffn;
+            if ((rc = ifa_glu_f32(1, n->proj + L.c_fg, NI, T, F, n->m3, F, s))) return rc;
+            if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_FFN_DOWN).data, W, F, n->m3, F, T, (const bf16_t *)L.T(IFA_LT_FFN_DOWN_B).data,
+                             (const bf16_t *)L.T(IFA_LT_LS2).data, 1.0f, 1, n->x, W))) return rc;
+        }
+        if (n->opt_tap_layers && n->taps && T <= n->taps_rows)
+            IFA_HIP_CHECK(hipMemcpyAsync(n->taps + li * n->taps_rows * W, n->x, T * W * 4, hipMemcpyDeviceToDevice, m->stream));
+    }
+    return IFA_OK;
+}
+
+// final norm + lm_head over rows [r0, r0 + nr) of the residual -> n->logits rows [0, nr)
+int run_head(ifa_model *m, size_t r0, size_t nr)
+{
+    LayeredNet *n = m->lay;
+    const size_t W = (size_t)n->cfg.width, V = (size_t)n->cfg.vocab;
+    int rc;
+    if ((rc = ifa_layernorm_f32(1, n->x + r0 * W, W, nr, W, n->out_norm.data, n->cfg.eps, n->h, W, (ifa_stream)m->stream))) return rc;
+    if ((rc = linear(m, (const bf16_t *)n->lm_head.data, V, W, n->h, W, nr, nullptr, nullptr, 1.0f, 0, n->logits, V))) return rc;
+    n->logits_rows = nr;
+    return IFA_OK;
+}
+
+__global__ void k_lay_advance(int *tokens, int *pos, ifa_seq_desc *seqs, const int *next, int *ring, int step)
+{
+    tokens[0] = next[0]; pos[0] += 1; seqs[0].pos0 += 1; ring[step] = next[0];
+}
+
+// ---- the worker class
+int lay_destroy(ifa_model *m)
+{
+    LayeredNet *n = m->lay;
+    (void)hipSetDevice(m->cfg.device);
+    if (m->stream) (void)hipStreamSynchronize(m->stream);
+    drop_step_graph(n);
+    for (LLayer &L : n->layers) {
+        for (LTensor &t : L.t) lay_free(t.data);
+        lay_free(L.w_in); lay_free(L.b_in); lay_free(L.w_conv); lay_free(L.bucket_of);
+    }
+    lay_free(n->embd.data); lay_free(n->out_norm.data); lay_free(n->lm_head.data);
+    for (float *p : n->slot_ptr) lay_free(p);
+    lay_free(n->slot_base_dev);
+    if (n->tab_pin) (void)hipHostFree(n->tab_pin);
+    lay_free(n->tab_dev); lay_free(n->excl_dev); lay_free(n->next_dev); lay_free(n->ring_dev);
+    float *bufs[] = {n->x, n->h, n->proj, n->m1, n->m2, n->m3, n->beta, n->decay, n->logits, n->taps};
+    for (float *b : bufs) lay_free(b);
+    if (m->stream && m->own_stream) (void)hipStreamDestroy(m->stream);
+    delete n;
+    delete m;
+    return IFA_OK;
+}
+
+int cat_rows(std::vector<bf16_t> &w, std::vector<bf16_t> &b, const LTensor &t, const LTensor *bias, size_t K, size_t &off, hipStream_t s)
+{
+    IFA_REQUIRE(t.present() && t.cols == K, "layer-list worker: a projection is missing or has %zu columns instead of %zu", t.cols, K);
+    off = b.size();
+    const size_t old = w.size();
+    w.resize(old + t.rows * K);
+    IFA_HIP_CHECK(hipMemcpy(w.data() + old, t.data, t.rows * K * 2, hipMemcpyDeviceToHost));
+    b.resize(off + t.rows, 0);
+    if (bias && bias->present()) IFA_HIP_CHECK(hipMemcpy(b.data() + off, bias->data, t.rows * 2, hipMemcpyDeviceToHost));
+    return IFA_OK;
+}
+
+int lay_finalize(ifa_model *m)
+{
+    LayeredNet *n = m->lay;
+    IFA_HIP_CHECK(hipSetDevice(m->cfg.device));
+    const size_t W = (size_t)n->cfg.width;
+    IFA_REQUIRE(n->embd.present() && n->out_norm.present() && n->lm_head.present(), "layer-list worker: embedding, final norm or lm_head is missing");
+    size_t off = 0;
+    n->n_in_max = n->mix_max = n->ffn_max = n->heads_max = 4;
+    for (size_t li = 0; li < n->layers.size(); li++) {
+        LLayer &L = n->layers[li];
+        const ifa_layer_spec &sp = L.spec;
+        if (L.w_in) continue;          // finalized before
+        for (int id = IFA_LT_NORM1; id < IFA_LT_END; id++) {
+            size_t r, c; bool vec;
+            if (expected_shape(n, sp, id, r, c, vec)) IFA_REQUIRE(L.T(id).present(), "layer-list worker: tensor %d of layer %zu is missing", id, li);
+        }
+        std::vector<bf16_t> w, b;
+        int rc;
+        if (sp.mixer == IFA_MIX_WINDOW_LINEAR) {
+            if ((rc = cat_rows(w, b, L.T(IFA_LT_A_Q), nullptr, W, L.c_aq, m->stream)) || (rc = cat_rows(w, b, L.T(IFA_LT_A_K), nullptr, W, L.c_ak, m->stream))
+                || (rc = cat_rows(w, b, L.T(IFA_LT_L_Q), nullptr, W, L.c_lq, m->stream)) || (rc = cat_rows(w, b, L.T(IFA_LT_L_K), nullptr, W, L.c_lk, m->stream))
+                || (rc = cat_rows(w, b, L.T(IFA_LT_L_V), nullptr, W, L.c_lv, m->stream)) || (rc = cat_rows(w, b, L.T(IFA_LT_L_G), nullptr, W, L.c_lg, m->stream))) return rc;
+            std::vector<int> bk;
+            build_buckets(bk, n->cfg.max_ctx, sp.a_buckets, sp.a_bias_max);
+            IFA_HIP_CHECK(hipMalloc((void **)&L.bucket_of, bk.size() * 4));
+            IFA_HIP_CHECK(hipMemcpy(L.bucket_of, bk.data(), bk.size() * 4, hipMemcpyHostToDevice));
+            const size_t kv = align4((size_t)n->cfg.max_ctx * sp.a_kv_heads * sp.a_dim);
+            L.o_k = off; off += kv; L.o_v = off; off += kv;
+            L.o_lin = off; off += align4((size_t)sp.l_heads * sp.l_dim * sp.l_vdim);
+            n->mix_max = std::max({n->mix_max, (size_t)sp.a_heads * sp.a_dim, (size_t)sp.l_heads * sp.l_vdim});
+            n->heads_max = std::max(n->heads_max, (size_t)std::max(sp.a_heads, sp.l_heads));
+        } else {
+            size_t dk_off, dv_off;
+            if ((rc = cat_rows(w, b, L.T(IFA_LT_D_Q), nullptr, W, L.c_dq, m->stream)) || (rc = cat_rows(w, b, L.T(IFA_LT_D_K), nullptr, W, dk_off, m->stream))
+                || (rc = cat_rows(w, b, L.T(IFA_LT_D_V), nullptr, W, dv_off, m->stream)) || (rc = cat_rows(w, b, L.T(IFA_LT_D_B), nullptr, W, L.c_db, m->stream))
+                || (rc = cat_rows(w, b, L.T(IFA_LT_D_A), nullptr, W, L.c_da, m->stream)) || (rc = cat_rows(w, b, L.T(IFA_LT_D_G), nullptr, W, L.c_dg, m->stream))) return rc;
+            const size_t QK = (size_t)sp.d_kv_heads * sp.d_dim, DV = (size_t)sp.d_heads * sp.d_vdim;
+            L.conv_ch = (int)(2 * QK + DV);
+            std::vector<bf16_t> cw((size_t)L.conv_ch * sp.d_conv);
+            IFA_HIP_CHECK(hipMemcpy(cw.data(), L.T(IFA_LT_D_QCONV).data, QK * sp.d_conv * 2, hipMemcpyDeviceToHost));
+            IFA_HIP_CHECK(hipMemcpy(cw.data() + QK * sp.d_conv, L.T(IFA_LT_D_KCONV).data, QK * sp.d_conv * 2, hipMemcpyDeviceToHost));
+            IFA_HIP_CHECK(hipMemcpy(cw.data() + 2 * QK * sp.d_conv, L.T(IFA_LT_D_VCONV).data, DV * sp.d_conv * 2, hipMemcpyDeviceToHost));
+            IFA_HIP_CHECK(hipMalloc((void **)&L.w_conv, cw.size() * 2));
+            IFA_HIP_CHECK(hipMemcpy(L.w_conv, cw.data(), cw.size() * 2, hipMemcpyHostToDevice));
+            L.o_rec = off; off += align4((size_t)sp.d_heads * sp.d_dim * sp.d_vdim);
+            L.o_conv = off; off += align4((size_t)std::max(sp.d_conv - 1, 0) * L.conv_ch);
+            n->mix_max = std::max({n->mix_max, (size_t)L.conv_ch, DV});
+            n->heads_max = std::max(n->heads_max, (size_t)sp.d_heads);
+        }
+        if (sp.ffn > 0) {
+            size_t up_off;
+            if ((rc = cat_rows(w, b, L.T(IFA_LT_FFN_GATE), &L.T(IFA_LT_FFN_GATE_B), W, L.c_fg, m->stream))
+                || (rc = cat_rows(w, b, L.T(IFA_LT_FFN_UP), &L.T(IFA_LT_FFN_UP_B), W, up_off, m->stream))) return rc;
+            n->ffn_max = std::max(n->ffn_max, (size_t)sp.ffn);
+        }
+        L.n_in = b.size();
+        // the product's row stride: a multiple of 4 floats so that every row of it starts 16-byte aligned
+        while (L.n_in % 4) { w.resize(w.size() + W, 0); b.push_back(0); L.n_in++; }
+        IFA_HIP_CHECK(hipMalloc((void **)&L.w_in, w.size() * 2));
+        IFA_HIP_CHECK(hipMalloc((void **)&L.b_in, b.size() * 2));
+        IFA_HIP_CHECK(hipMemcpy(L.w_in, w.data(), w.size() * 2, hipMemcpyHostToDevice));
+        IFA_HIP_CHECK(hipMemcpy(L.b_in, b.data(), b.size() * 2, hipMemcpyHostToDevice));
+        n->n_in_max = std::max(n->n_in_max, L.n_in);
+        // the separate copies of what the fused product now holds are no longer needed
+        for (int id : {IFA_LT_A_Q, IFA_LT_A_K, IFA_LT_L_Q, IFA_LT_L_K, IFA_LT_L_V, IFA_LT_L_G, IFA_LT_D_Q, IFA_LT_D_K, IFA_LT_D_V, IFA_LT_D_B, IFA_LT_D_A,
+                       IFA_LT_D_G, IFA_LT_FFN_GATE, IFA_LT_FFN_UP}) {
+            LTensor &t = L.T(id);
+            if (t.data) { lay_free(t.data); t.data = nullptr; }
+        }
+    }
+    if (!n->slot_base_dev) {
+        n->arena_floats = off;
+        n->slot_ptr.assign((size_t)MAX_SLOTS, nullptr);
+        IFA_HIP_CHECK(hipMalloc((void **)&n->slot_base_dev, sizeof(float *) * MAX_SLOTS));
+        IFA_HIP_CHECK(hipMemset(n->slot_base_dev, 0, sizeof(float *) * MAX_SLOTS));
+        IFA_HIP_CHECK(hipMalloc((void **)&n->excl_dev, 4 * sizeof(int)));
+        IFA_HIP_CHECK(hipMemset(n->excl_dev, 0, 4 * sizeof(int)));
+        IFA_HIP_CHECK(hipMalloc((void **)&n->next_dev, sizeof(int) * ifa_model::RING));
+        IFA_HIP_CHECK(hipMalloc((void **)&n->ring_dev, sizeof(int) * ifa_model::RING));
+    }
+    m->finalized = true;
+    return IFA_OK;
+}
+
+int lay_reset(ifa_model *m) { IFA_REQUIRE(m->finalized, "ifa_model_reset: model not finalized"); return IFA_OK; }      // (position 0 restarts every state)
+
+int lay_kv_slots(ifa_model *m, int n_slots)
+{
+    IFA_REQUIRE(m->finalized, "ifa_model_kv_slots: model not finalized");
+    IFA_REQUIRE(n_slots >= 1 && n_slots <= MAX_SLOTS, "ifa_model_kv_slots: n_slots %d", n_slots);
+    IFA_REQUIRE(n_slots >= m->lay->n_slots, "ifa_model_kv_slots: cannot shrink below %d slots", m->lay->n_slots);
+    m->lay->n_slots = n_slots;
+    return IFA_OK;
+}
+
+int lay_select_kv(ifa_model *m, int slot)
+{
+    IFA_REQUIRE(m->finalized, "ifa_model_select_kv: model not finalized");
+    IFA_REQUIRE(slot >= 0 && slot < m->lay->n_slots, "ifa_model_select_kv: slot %d of %d", slot, m->lay->n_slots);
+    m->lay->cur_slot = slot; m->cur_slot = slot;
+    return IFA_OK;
+}
+
+int lay_set_option(ifa_model *m, const char *name, int value)
+{
+    LayeredNet *n = m->lay;
+    if (!strcmp(name, "tap_layers")) { n->opt_tap_layers = value; drop_step_graph(n); return IFA_OK; }
+    if (!strcmp(name, "graph")) { n->opt_graph = value; drop_step_graph(n); return IFA_OK; }
+    if (!strcmp(name, "ops32")) { IFA_HIP_CHECK(hipStreamSynchronize(m->stream)); n->cfg.ops32 = value ? 1 : 0; drop_step_graph(n); return IFA_OK; }
+    return ifa_fail(IFA_ERR_ARG, "ifa_model_set_option: unknown option '%s' (layer-list model: tap_layers, graph, ops32)", name);
+}
+
+int lay_set_excluded(ifa_model *m, const int *ids_host, int cnt)
+{
+    IFA_REQUIRE(m->finalized, "ifa_model_set_excluded_tokens: model not finalized");
+    IFA_REQUIRE(cnt >= 0 && cnt <= 3 && (cnt == 0 || ids_host), "ifa_model_set_excluded_tokens: n %d (0..3)", cnt);
+    int v[4] = {cnt, -1, -1, -1};
+    for (int i = 0; i < cnt; i++) v[1 + i] = ids_host[i];
+    IFA_HIP_CHECK(hipStreamSynchronize(m->stream));
+    IFA_HIP_CHECK(hipMemcpy(m->lay->excl_dev, v, sizeof(v), hipMemcpyHostToDevice));
+    return IFA_OK;
+}
+
+int lay_get_buffer(ifa_model *m, const char *name, int layer, void **dptr, size_t *bytes)
+{
+    LayeredNet *n = m->lay;
+    size_t b = 0; void *p = nullptr;
+    if (!strcmp(name, "logits")) { p = n->logits; b = n->logits_rows * (size_t)n->cfg.vocab * 4; }
+    else if (!strcmp(name, "x")) { p = n->x; b = n->scratch_rows * (size_t)n->cfg.width * 4; }
+    else if (!strcmp(name, "layer_taps")) {      // [layers][taps_rows][width] fp32: the residual after every layer of the last step (option tap_layers)
+        IFA_REQUIRE(n->taps, "ifa_model_get_buffer: no taps (set option tap_layers before the step)");
+        IFA_REQUIRE(layer >= 0 && layer < (int)n->layers.size(), "ifa_model_get_buffer: layer %d", layer);
+        p = n->taps + (size_t)layer * n->taps_rows * n->cfg.width; b = n->taps_rows * (size_t)n->cfg.width * 4;
+    } else if (!strcmp(name, "slot")) {          // the arena of slot `layer`
+        IFA_REQUIRE(layer >= 0 && layer < n->n_slots, "ifa_model_get_buffer: slot %d", layer);
+        p = n->slot_ptr[(size_t)layer]; b = p ? n->arena_floats * 4 : 0;
+    } else return ifa_fail(IFA_ERR_ARG, "ifa_model_get_buffer: unknown buffer '%s'", name);
+    *dptr = p;
+    if (bytes) *bytes = b;
+    return IFA_OK;
+}
+
+// tables of a step -> device
+int upload_tables(ifa_model *m, const std::vector<int> &tokens, const std::vector<int> &pos, const std::vector<int> &row_seq, const std::vector<ifa_seq_desc> &seqs)
+{
+    LayeredNet *n = m->lay;
+    const size_t T = tokens.size(), S = seqs.size(), R = n->tab_rows;
+    memcpy(n->tab_pin, tokens.data(), T * 4);
+    memcpy(n->tab_pin + R, pos.data(), T * 4);
+    memcpy(n->tab_pin + 2 * R, row_seq.data(), T * 4);
+    memcpy(n->tab_pin + 3 * R, seqs.data(), S * sizeof(ifa_seq_desc));
+    IFA_HIP_CHECK(hipMemcpyAsync(n->tab_dev, n->tab_pin, (3 * R + 4 * S) * 4, hipMemcpyHostToDevice, m->stream));
+    return IFA_OK;
+}
+
+int check_span(ifa_model *m, int n_tokens, int start, const int *tokens)
+{
+    const ifa_layered_config &c = m->lay->cfg;
+    IFA_REQUIRE(n_tokens >= 1 && start >= 0 && start + n_tokens <= c.max_ctx, "layer-list worker: tokens [%d, %d) exceed the context of %d", start, start + n_tokens, c.max_ctx);
+    for (int i = 0; tokens && i < n_tokens; i++) IFA_REQUIRE(tokens[i] >= 0 && tokens[i] < c.vocab, "layer-list worker: token id %d out of range", tokens[i]);
+    return IFA_OK;
+}
+
+int ensure_taps(ifa_model *m, size_t T)
+{
+    LayeredNet *n = m->lay;
+    if (!n->opt_tap_layers || T <= n->taps_rows) return IFA_OK;
+    IFA_HIP_CHECK(hipStreamSynchronize(m->stream));
+    lay_free(n->taps); n->taps = nullptr;
+    IFA_HIP_CHECK(hipMalloc((void **)&n->taps, n->layers.size() * T * (size_t)n->cfg.width * 4));
+    n->taps_rows = T;
+    return IFA_OK;
+}
+
+// One step over several sequences: sequence q brings lens[q] tokens (concatenated in tokens_host) at positions [pos0[q], pos0[q] + lens[q])
+// of the query in slot slots[q].  logits_mode 0: only the last row of every sequence goes through the head (rows of n->logits = sequences),
+// 1: every row does.  next_tokens_host[q] = greedy token after the last row of sequence q.
+int lay_step(ifa_model *m, int nseq, const int *tokens_host, const int *lens, const int *pos0, const int *slots, int logits_mode, int *next_tokens_host)
+{
+    LayeredNet *n = m->lay;
+    IFA_REQUIRE(nseq >= 1 && nseq <= ifa_model::RING && tokens_host && lens && pos0 && slots, "layer-list step: bad arguments");
+    IFA_HIP_CHECK(hipSetDevice(m->cfg.device));
+    int rc;
+    size_t T = 0;
+    for (int q = 0; q < nseq; q++) {
+        if ((rc = check_span(m, lens[q], pos0[q], tokens_host + T)) || (rc = ensure_slot(m, slots[q]))) return rc;
+        for (int b = 0; b < q; b++) IFA_REQUIRE(slots[q] != slots[b], "layer-list step: slot %d used twice", slots[q]);
+        T += (size_t)lens[q];
+    }
+    const size_t V = (size_t)n->cfg.vocab, W = (size_t)n->cfg.width;
+    const bool all = logits_mode != 0 || T == (size_t)nseq;
+    if ((rc = ensure_rows(m, T, (size_t)nseq)) || (rc = ensure_taps(m, T)) || (rc = ensure_logits(m, all ? T : (size_t)nseq))) return rc;
+    std::vector<int> tok(tokens_host, tokens_host + T), pos(T), rs(T), last((size_t)nseq);
+    std::vector<ifa_seq_desc> sq((size_t)nseq);
+    size_t r = 0;
+    for (int q = 0; q < nseq; q++) {
+        sq[(size_t)q] = ifa_seq_desc{(int)r, lens[q], pos0[q], slots[q]};
+        for (int i = 0; i < lens[q]; i++, r++) { pos[r] = pos0[q] + i; rs[r] = q; }
+        last[(size_t)q] = (int)r - 1;
+    }
+    if ((rc = upload_tables(m, tok, pos, rs, sq)) || (rc = run_layers(m, T, nseq))) return rc;
+    ifa_stream s = (ifa_stream)m->stream;
+    if (all) {
+        if ((rc = run_head(m, 0, T))) return rc;
+        for (int q = 0; q < nseq; q++)
+            if ((rc = ifa_argmax_rows_f32(n->logits + (size_t)last[(size_t)q] * V, V, V, 1, n->excl_dev, n->next_dev + q, s))) return rc;
+    } else {
+        // the sequences' last rows, normed one by one into consecutive rows of h, then one product
+        for (int q = 0; q < nseq; q++)
+            if ((rc = ifa_layernorm_f32(1, n->x + (size_t)last[(size_t)q] * W, W, 1, W, n->out_norm.data, n->cfg.eps, n->h + (size_t)q * W, W, s))) return rc;
+        if ((rc = linear(m, (const bf16_t *)n->lm_head.data, V, W, n->h, W, (size_t)nseq, nullptr, nullptr, 1.0f, 0, n->logits, V))) return rc;
+        n->logits_rows = (size_t)nseq;
+        if ((rc = ifa_argmax_rows_f32(n->logits, V, V, (size_t)nseq, n->excl_dev, n->next_dev, s))) return rc;
+    }
+    std::vector<int> next((size_t)nseq, -1);
+    IFA_HIP_CHECK(hipMemcpyAsync(next.data(), n->next_dev, (size_t)nseq * 4, hipMemcpyDeviceToHost, m->stream));
+    IFA_HIP_CHECK(hipStreamSynchronize(m->stream));
+    if (next_tokens_host) memcpy(next_tokens_host, next.data(), (size_t)nseq * 4);
+    return IFA_OK;
+}
+
+int lay_forward(ifa_model *m, const int *tokens_host, int n_tokens, int prefix_len, void *logits_out_dev, int *next_token_host)
+{
+    LayeredNet *n = m->lay;
+    IFA_REQUIRE(tokens_host, "ifa_model_forward: null tokens");
+    int rc = lay_step(m, 1, tokens_host, &n_tokens, &prefix_len, &n->cur_slot, logits_out_dev ? 1 : 0, next_token_host);
+    if (rc || !logits_out_dev) return rc;
+    if ((rc = ifa_convert_f32_f16(n->logits, (size_t)n_tokens * n->cfg.vocab, logits_out_dev, (ifa_stream)m->stream))) return rc;
+    IFA_HIP_CHECK(hipStreamSynchronize(m->stream));
+    return IFA_OK;
+}
+
+int lay_decode_batch(ifa_model *m, int cnt, const int *tokens_host, const int *positions_host, const int *kv_slots_host, int *next_tokens_host,
+                     void *logits_out_dev)
+{
+    LayeredNet *n = m->lay;
+    IFA_REQUIRE(cnt >= 1 && cnt <= ifa_model::RING, "ifa_model_decode_batch: bad arguments");
+    std::vector<int> ones((size_t)cnt, 1);
+    int rc = lay_step(m, cnt, tokens_host, ones.data(), positions_host, kv_slots_host, 1, next_tokens_host);
+    if (rc || !logits_out_dev) return rc;
+    if ((rc = ifa_convert_f32_f16(n->logits, (size_t)cnt * n->cfg.vocab, logits_out_dev, (ifa_stream)m->stream))) return rc;
+    IFA_HIP_CHECK(hipStreamSynchronize(m->stream));
+    return IFA_OK;
+}
+
+// one token of the current slot's sequence, everything it depends on in device memory: capturable
+int enqueue_decode_step(ifa_model *m)
+{
+    LayeredNet *n = m->lay;
+    const size_t V = (size_t)n->cfg.vocab;
+    int rc;
+    if ((rc = run_layers(m, 1, 1)) || (rc = run_head(m, 0, 1))) return rc;
+    return ifa_argmax_rows_f32(n->logits, V, V, 1, n->excl_dev, n->next_dev, (ifa_stream)m->stream);
+}
+
+int lay_decode(ifa_model *m, int first_token, int start_pos, int n_steps, int *out_tokens_host, float *elapsed_ms, bool prepare_only)
+{
+    LayeredNet *n = m->lay;
+    IFA_REQUIRE(m->finalized, "ifa_model_decode: model not finalized");
+    IFA_REQUIRE(n_steps >= 1 && n_steps <= ifa_model::RING, "ifa_model_decode: n_steps %d (1..%d)", n_steps, ifa_model::RING);
+    IFA_HIP_CHECK(hipSetDevice(m->cfg.device));
+    int rc;
+    if ((rc = check_span(m, n_steps, start_pos, nullptr)) || (rc = ensure_slot(m, n->cur_slot)) || (rc = ensure_rows(m, 1, 1)) || (rc = ensure_logits(m, 1))) return rc;
+    if (n->opt_graph && !n->opt_tap_layers && !n->step_exec) {      // (the slot is read from the device tables: one capture serves every slot)
+        drop_step_graph(n);
+        IFA_HIP_CHECK(hipStreamSynchronize(m->stream));
+        IFA_HIP_CHECK(hipStreamBeginCapture(m->stream, hipStreamCaptureModeThreadLocal));
+        rc = enqueue_decode_step(m);
+        hipGraph_t g = nullptr;
+        const hipError_t e = hipStreamEndCapture(m->stream, &g);
+        if (rc) { if (g) (void)hipGraphDestroy(g); return rc; }
+        if (e != hipSuccess) return ifa_fail(IFA_ERR_HIP, "capture of the decode step: %s", hipGetErrorString(e));
+        n->step_graph = g;
+        IFA_HIP_CHECK(hipGraphInstantiate(&n->step_exec, g, nullptr, nullptr, 0));
+        n->step_slot = n->cur_slot;
+    }
+    if (prepare_only) return IFA_OK;
+    IFA_REQUIRE(out_tokens_host, "ifa_model_decode: null output");
+    if ((rc = check_span(m, 1, start_pos, &first_token))) return rc;
+    std::vector<int> tok(1, first_token), pos(1, start_pos), rs(1, 0);
+    std::vector<ifa_seq_desc> sq(1); sq[0] = ifa_seq_desc{0, 1, start_pos, n->cur_slot};
+    if ((rc = upload_tables(m, tok, pos, rs, sq))) return rc;
+    hipEvent_t e0 = nullptr, e1 = nullptr;
+    if (elapsed_ms) { IFA_HIP_CHECK(hipEventCreate(&e0)); IFA_HIP_CHECK(hipEventCreate(&e1)); IFA_HIP_CHECK(hipEventRecord(e0, m->stream)); }
+    for (int st = 0; st < n_steps; st++) {
+        if (n->step_exec && n->opt_graph && !n->opt_tap_layers) IFA_HIP_CHECK(hipGraphLaunch(n->step_exec, m->stream));
+        else if ((rc = enqueue_decode_step(m))) return rc;
+        hipLaunchKernelGGL(k_lay_advance, dim3(1), dim3(1), 0, m->stream, n->tokens_dev, n->pos_dev, n->seqs_dev, n->next_dev, n->ring_dev, st);
+        IFA_LAUNCH_CHECK();
+    }
+    if (elapsed_ms) IFA_HIP_CHECK(hipEventRecord(e1, m->stream));
+    IFA_HIP_CHECK(hipMemcpyAsync(out_tokens_host, n->ring_dev, (size_t)n_steps * 4, hipMemcpyDeviceToHost, m->stream));
+    IFA_HIP_CHECK(hipStreamSynchronize(m->stream));
+    if (elapsed_ms) { IFA_HIP_CHECK(hipEventElapsedTime(elapsed_ms, e0, e1)); (void)hipEventDestroy(e0); (void)hipEventDestroy(e1); }
+    return IFA_OK;
+}
+
+const ifa_model_vtbl kLayeredVtbl = {lay_destroy, lay_finalize, lay_reset, lay_kv_slots, lay_select_kv, lay_set_option, lay_set_excluded, lay_get_buffer,
+                                     lay_forward, lay_decode, lay_decode_batch};
+
+} // namespace
+
+extern "C" {
+
+int ifa_model_create_layered(const ifa_layered_config *cfg, const ifa_layer_spec *layers, ifa_model **out)
+{
+    IFA_REQUIRE(cfg && layers && out, "ifa_model_create_layered: null pointer");
+    IFA_REQUIRE(cfg->width > 0 && cfg->vocab > 0 && cfg->max_ctx > 0 && cfg->n_layers > 0, "ifa_model_create_layered: bad hyper-parameters");
+    for (int l = 0; l < cfg->n_layers; l++) {
+        const ifa_layer_spec &s = layers[l];
+        IFA_REQUIRE(s.ffn >= 0, "ifa_model_create_layered: layer %d: ffn %d", l, s.ffn);
+        if (s.mixer == IFA_MIX_WINDOW_LINEAR) {
+            IFA_REQUIRE(s.a_heads > 0 && s.a_kv_heads > 0 && s.a_heads % s.a_kv_heads == 0 && s.a_dim > 0 && s.a_dim <= 256 && s.a_window >= 1 && s.a_keep_first >= 0
+                        && s.a_buckets >= 1 && s.a_bias_max >= 1, "ifa_model_create_layered: layer %d: bad windowed-attention sizes", l);
+            IFA_REQUIRE(s.l_heads > 0 && s.l_dim > 0 && s.l_dim <= 256 && s.l_vdim > 0, "ifa_model_create_layered: layer %d: bad linear-attention sizes", l);
+        } else if (s.mixer == IFA_MIX_GATED_DELTA) {
+            IFA_REQUIRE(s.d_heads > 0 && s.d_kv_heads > 0 && s.d_heads % s.d_kv_heads == 0 && s.d_dim > 0 && s.d_dim <= 256 && s.d_vdim > 0 && s.d_conv >= 1 && s.d_conv <= 64,
+                        "ifa_model_create_layered: layer %d: bad delta-rule sizes", l);
+            IFA_REQUIRE((2 * (size_t)s.d_kv_heads * s.d_dim + (size_t)s.d_heads * s.d_vdim) * 4 <= 64 * 1024, "ifa_model_create_layered: layer %d: the convolution's channels do not fit one LDS row", l);
+        } else return ifa_fail(IFA_ERR_ARG, "ifa_model_create_layered: layer %d: unknown mixer %d", l, s.mixer);
+    }
+    IFA_HIP_CHECK(hipSetDevice(cfg->device));
+    ifa_model *m = new ifa_model();
+    memset(&m->cfg, 0, sizeof(m->cfg));
+    m->cfg.dim = cfg->width; m->cfg.layers = cfg->n_layers; m->cfg.vocab = cfg->vocab; m->cfg.max_ctx = cfg->max_ctx; m->cfg.device = cfg->device;
+    m->cfg.eps = cfg->eps; m->cfg.tp_size = 1;
+    LayeredNet *n = new LayeredNet();
+    n->cfg = *cfg;
+    if (n->cfg.eps <= 0) n->cfg.eps = 1e-5f;
+    if (n->cfg.pos_base <= 1.0f) n->cfg.pos_base = 10000.0f;
+    n->layers.resize((size_t)cfg->n_layers);
+    for (int l = 0; l < cfg->n_layers; l++) n->layers[(size_t)l].spec = layers[l];
+    m->lay = n; m->vt = &kLayeredVtbl;
+    hipError_t e = hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking);
+    if (e != hipSuccess) { delete n; delete m; return ifa_fail(IFA_ERR_HIP, "hipStreamCreate: %s", hipGetErrorString(e)); }
+    *out = m;
+    return IFA_OK;
+}
+
+int ifa_model_set_tensor_host(ifa_model *m, int layer, int tensor_id, int dtype, const void *host_src, size_t rows, size_t cols)
+{
+    IFA_REQUIRE(m && m->lay && host_src, "ifa_model_set_tensor_host: not a layer-list model / null pointer");
+    LayeredNet *n = m->lay;
+    IFA_REQUIRE(!m->finalized, "ifa_model_set_tensor_host: the model is finalized");
+    IFA_REQUIRE(rows > 0 && cols > 0, "ifa_model_set_tensor_host: empty tensor");
+    LTensor *t = nullptr;
+    size_t er = 0, ec = 0; bool vec = false;
+    const size_t W = (size_t)n->cfg.width, V = (size_t)n->cfg.vocab;
+    if (layer < 0) {
+        if (tensor_id == IFA_T_EMBD) { t = &n->embd; er = V; ec = W; }
+        else if (tensor_id == IFA_T_LM_HEAD) { t = &n->lm_head; er = V; ec = W; }
+        else if (tensor_id == IFA_T_OUT_NORM) { t = &n->out_norm; er = 1; ec = W; vec = true; }
+        else return ifa_fail(IFA_ERR_ARG, "ifa_model_set_tensor_host: global tensor id %d", tensor_id);
+    } else {
+        IFA_REQUIRE(layer < (int)n->layers.size() && tensor_id >= IFA_LT_NORM1 && tensor_id < IFA_LT_END, "ifa_model_set_tensor_host: layer %d / tensor id %d", layer, tensor_id);
+        LLayer &L = n->layers[(size_t)layer];
+        IFA_REQUIRE(expected_shape(n, L.spec, tensor_id, er, ec, vec), "ifa_model_set_tensor_host: tensor %d does not belong to layer %d's mixer", tensor_id, layer);
+        t = &L.T(tensor_id);
+    }
+    const int want = tensor_id == IFA_LT_L_DECAY ? IFA_F32 : IFA_BF16;
+    IFA_REQUIRE(dtype == want, "ifa_model_set_tensor_host: tensor %d takes dtype %d, got %d", tensor_id, want, dtype);
+    if (vec) IFA_REQUIRE(rows * cols == er * ec, "ifa_model_set_tensor_host: tensor %d of layer %d holds %zu values, the model needs %zu", tensor_id, layer, rows * cols, er * ec);
+    else IFA_REQUIRE(rows == er && cols == ec, "ifa_model_set_tensor_host: tensor %d of layer %d is %zu x %zu, the model needs %zu x %zu", tensor_id, layer, rows, cols, er, ec);
+    IFA_HIP_CHECK(hipSetDevice(m->cfg.device));
+    lay_free(t->data); t->data = nullptr;
+    const size_t bytes = rows * cols * (dtype == IFA_F32 ? 4 : 2);
+    IFA_HIP_CHECK(hipMalloc(&t->data, bytes));
+    IFA_HIP_CHECK(hipMemcpy(t->data, host_src, bytes, hipMemcpyHostToDevice));
+    t->dtype = dtype; t->rows = rows; t->cols = cols;
+    return IFA_OK;
+}
+
+int ifa_model_logits_f32(ifa_model *m, void **dptr, size_t *rows, size_t *cols)
+{
+    IFA_REQUIRE(m && m->lay && dptr, "ifa_model_logits_f32: not a layer-list model / null pointer");
+    *dptr = m->lay->logits;
+    if (rows) *rows = m->lay->logits_rows;
+    if (cols) *cols = (size_t)m->lay->cfg.vocab;
+    return IFA_OK;
+}
+
+int ifa_model_step_seqs(ifa_model *m, int n_seqs, const int *tokens_host, const int *seq_lens, const int *seq_pos0, const int *seq_slots, int all_logits,
+                        int *next_tokens_host)
+{
+    IFA_REQUIRE(m && m->lay && m->finalized, "ifa_model_step_seqs: not a finalized layer-list model");
+    return lay_step(m, n_seqs, tokens_host, seq_lens, seq_pos0, seq_slots, all_logits, next_tokens_host);
+}
+
+int ifa_model_is_layered(const ifa_model *m) { return m && m->vt ? 1 : 0; }
+
+} // extern "C"

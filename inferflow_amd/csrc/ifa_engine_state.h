@@ -62,8 +62,30 @@ struct Layer {
 } // namespace ifae
 using namespace ifae;
 
+// A second worker class behind the same ifa_model handle (the layer-list worker, ifa_engine_layered.hip): when `vt` is set, the
+// ifa_model_* entry points that both classes answer hand the call to it; the entry points of the standard network's own machinery
+// (tensor-parallel seams, kernel timing, per-phase statistics) decline.
+struct ifa_model;
+struct ifa_model_vtbl {
+    int (*destroy)(ifa_model *m);
+    int (*finalize)(ifa_model *m);
+    int (*reset)(ifa_model *m);
+    int (*kv_slots)(ifa_model *m, int n_slots);
+    int (*select_kv)(ifa_model *m, int slot);
+    int (*set_option)(ifa_model *m, const char *name, int value);
+    int (*set_excluded_tokens)(ifa_model *m, const int *ids_host, int n);
+    int (*get_buffer)(ifa_model *m, const char *name, int layer, void **dptr, size_t *bytes);
+    int (*forward)(ifa_model *m, const int *tokens_host, int n_tokens, int prefix_len, void *logits_out_dev, int *next_token_host);
+    int (*decode)(ifa_model *m, int first_token, int start_pos, int n_steps, int *out_tokens_host, float *elapsed_ms, bool prepare_only);
+    int (*decode_batch)(ifa_model *m, int n, const int *tokens_host, const int *positions_host, const int *kv_slots_host, int *next_tokens_host,
+                        void *logits_out_dev);
+};
+struct LayeredNet;
+
 struct ifa_model {
     ifa_model_config cfg;
+    const ifa_model_vtbl *vt = nullptr;     // null: the standard network of this file
+    LayeredNet *lay = nullptr;              // state of the layer-list worker
     std::vector<Layer> layers;
     Tensor g[10];
     hipStream_t stream = nullptr;
@@ -205,6 +227,9 @@ static inline bool scale_on(float s) { return s < 0.9999f || s > 1.0001f; }     
 // same tiled layout and arithmetic (the A/B variants differ only in how the quantizer picked base/scale)
 static inline bool same_fmt(int a, int b) { return a == b || (is_q4(a) && is_q4(b)); }
 
+
+// entry points only the standard network has
+#define IFA_STD_ONLY(m, who) do { if ((m) && (m)->vt) return ifa_fail(IFA_ERR_STATE, who ": not available for a layer-list model"); } while (0)
 
 static constexpr size_t IFA_LDS_LIMIT = 160 * 1024;      // LDS per workgroup on gfx950 (MI355X_MICROARCH.md)
 

@@ -143,6 +143,7 @@ extern "C" {
 
 int ifa_model_tp_begin(ifa_model *m, int token, int pos)
 {
+    IFA_STD_ONLY(m, "ifa_model_tp_begin");
     int rc = tp_ready(m);
     if (rc) return rc;
     m->pend.on = false;
@@ -159,6 +160,7 @@ int ifa_model_tp_begin(ifa_model *m, int token, int pos)
 
 int ifa_model_tp_begin_hidden(ifa_model *m, const void *x_f16, int pos)
 {
+    IFA_STD_ONLY(m, "ifa_model_tp_begin_hidden");
     int rc = tp_ready(m);
     if (rc) return rc;
     IFA_REQUIRE(x_f16, "ifa_model_tp_begin_hidden: null input");
@@ -175,6 +177,7 @@ int ifa_model_tp_begin_hidden(ifa_model *m, const void *x_f16, int pos)
 
 int ifa_model_tp_hidden(ifa_model *m, void *x_out_f16)
 {
+    IFA_STD_ONLY(m, "ifa_model_tp_hidden");
     IFA_REQUIRE(m && m->finalized && x_out_f16, "ifa_model_tp_hidden: bad arguments");
     { int rcf = tp_flush_pending(m); if (rcf) return rcf; }
     IFA_HIP_CHECK(hipMemcpyAsync(x_out_f16, m->x, (size_t)m->cfg.dim * 2, hipMemcpyDeviceToDevice, m->stream));
@@ -183,6 +186,7 @@ int ifa_model_tp_hidden(ifa_model *m, void *x_out_f16)
 
 int ifa_model_tp_attn(ifa_model *m, int layer, void *partial_out_f16)
 {
+    IFA_STD_ONLY(m, "ifa_model_tp_attn");
     IFA_REQUIRE(m && partial_out_f16 && layer >= 0 && layer < m->cfg.layers, "ifa_model_tp_attn: bad arguments");
     int rc;
     if ((rc = launch_qkv(m, layer, m->x))) return rc;
@@ -215,6 +219,7 @@ extern "C" {
 
 int ifa_model_tp_post_attn(ifa_model *m, int layer, const void *reduced_f16)
 {
+    IFA_STD_ONLY(m, "ifa_model_tp_post_attn");
     IFA_REQUIRE(m && reduced_f16 && layer >= 0 && layer < m->cfg.layers, "ifa_model_tp_post_attn: bad arguments");
     const size_t D = (size_t)m->cfg.dim;
     const Tensor &b = m->layers[(size_t)layer].t[T_WO_B];
@@ -246,6 +251,7 @@ int ifa_model_tp_post_attn(ifa_model *m, int layer, const void *reduced_f16)
 
 int ifa_model_tp_ffn(ifa_model *m, int layer, void *partial_out_f16)
 {
+    IFA_STD_ONLY(m, "ifa_model_tp_ffn");
     IFA_REQUIRE(m && partial_out_f16 && layer >= 0 && layer < m->cfg.layers, "ifa_model_tp_ffn: bad arguments");
     int rc;
     Layer &L = m->layers[(size_t)layer];
@@ -263,6 +269,7 @@ int ifa_model_tp_ffn(ifa_model *m, int layer, void *partial_out_f16)
 
 int ifa_model_tp_post_ffn(ifa_model *m, int layer, const void *reduced_f16)
 {
+    IFA_STD_ONLY(m, "ifa_model_tp_post_ffn");
     IFA_REQUIRE(m && reduced_f16 && layer >= 0 && layer < m->cfg.layers, "ifa_model_tp_post_ffn: bad arguments");
     const size_t D = (size_t)m->cfg.dim;
     const Tensor &b = m->layers[(size_t)layer].t[T_W2_B];
@@ -295,6 +302,7 @@ int ifa_model_tp_post_ffn(ifa_model *m, int layer, const void *reduced_f16)
 
 int ifa_model_tp_logits(ifa_model *m, void *logits_shard_out_f16)
 {
+    IFA_STD_ONLY(m, "ifa_model_tp_logits");
     IFA_REQUIRE(m && logits_shard_out_f16, "ifa_model_tp_logits: bad arguments");
     IFA_REQUIRE(m->g[T_LM_HEAD].present(), "ifa_model_tp_logits: this worker holds no lm_head (not the last pipeline stage)");
     { int rcf = tp_flush_pending(m); if (rcf) return rcf; }
@@ -303,6 +311,7 @@ int ifa_model_tp_logits(ifa_model *m, void *logits_shard_out_f16)
 
 int ifa_model_tp_set_token(ifa_model *m, const int *token_dev)
 {
+    IFA_STD_ONLY(m, "ifa_model_tp_set_token");
     IFA_REQUIRE(m && token_dev, "ifa_model_tp_set_token: bad arguments");
     k_tp_set_token<<<1, 1, 0, m->stream>>>(m->state, token_dev, ifa_model::RING);
     IFA_LAUNCH_CHECK();
@@ -403,6 +412,7 @@ extern "C" {
 int ifa_model_tp_prefill(ifa_model *m, const ifa_tp_topology *topo, const int *tokens_host, int n_tokens, int start_pos,
                          void *logits_shard_out_dev, int *next_token_host)
 {
+    IFA_STD_ONLY(m, "ifa_model_tp_prefill");
     IFA_REQUIRE(tokens_host && n_tokens >= 1, "ifa_model_tp_prefill: no tokens");
     int rc = tp_check(m, topo, "ifa_model_tp_prefill");
     if (rc) return rc;
@@ -437,6 +447,7 @@ int ifa_model_tp_prefill(ifa_model *m, const ifa_tp_topology *topo, const int *t
 int ifa_model_tp_decode_batch(ifa_model *m, const ifa_tp_topology *topo, int n, const int *tokens_host, const int *positions_host,
                               const int *kv_slots_host, int *next_tokens_host, void *logits_shard_out_dev)
 {
+    IFA_STD_ONLY(m, "ifa_model_tp_decode_batch");
     IFA_REQUIRE(n >= 1 && n <= ifa_model::RING && tokens_host && positions_host && kv_slots_host, "ifa_model_tp_decode_batch: bad arguments");
     int rc = tp_check(m, topo, "ifa_model_tp_decode_batch");
     if (rc) return rc;
@@ -450,6 +461,7 @@ int ifa_model_tp_decode_batch(ifa_model *m, const ifa_tp_topology *topo, int n, 
 int ifa_model_tp_decode(ifa_model *m, const ifa_tp_topology *topo, int first_token, int start_pos, int n_steps,
                         int *out_tokens_host, float *elapsed_ms)
 {
+    IFA_STD_ONLY(m, "ifa_model_tp_decode");
     IFA_REQUIRE(out_tokens_host, "ifa_model_tp_decode: null pointer");
     IFA_REQUIRE(n_steps >= 1 && n_steps <= ifa_model::RING, "ifa_model_tp_decode: n_steps %d (1..%d)", n_steps, ifa_model::RING);
     int rc = tp_check(m, topo, "ifa_model_tp_decode");

@@ -1,0 +1,201 @@
+// ifa_linear_bf16.hip -- linear layers with bfloat16 weights [N][K] and 32-bit activations [T][K]:
+//   C[t][n] (+)= alpha * mul[n] * (sum_k A[t][k] W[n][k] + bias[n])        (mul, bias optional; C in 32-bit floats)
+// The epilogue covers a plain projection (store), a projection with bias, and the residual update of a layer
+// (accumulate into the 32-bit residual stream with a per-channel layer scale and a branch scale).
+//
+//   T <= 8    k_lin_rows: one wave per output row, the weight row streamed once in 16-byte pieces, all T activation rows
+//             multiplied against it in fp32 (decode steps: bound by the weight stream)
+//   T  > 8    k_lin_mfma: 64 x 64 output tiles, K in steps of 32 through LDS, four waves of 32 x 32 sub-tiles;
+//             OPS32 = false: operands rounded to bfloat16, v_mfma_f32_32x32x16_bf16;
+//             OPS32 = true : operands stay 32-bit, v_mfma_f32_32x32x2_f32 (the exact mode of the worker)
+// Accumulation is fp32 in every path.  No atomics, no split K: a result does not depend on what else runs.
+#include "ifa_host.h"
+#include "ifa_f32_common.h"
+
+using namespace ifa32;
+
+namespace {
+
+typedef float f32x16v __attribute__((ext_vector_type(16)));
+typedef __bf16 bf16x8v __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
+
+struct LinArgs {
+    const bf16_t *W; const float *A; float *C;
+    const bf16_t *bias, *mul;
+    int T, N, K, lda, ldc;
+    float alpha; int accumulate, vec;
+};
+
+__device__ __forceinline__ void lin_store(const LinArgs &P, int t, int n, float acc)
+{
+    if (P.bias) acc += bf2f(P.bias[n]);
+    if (P.mul) acc *= bf2f(P.mul[n]);
+    acc *= P.alpha;
+    float *c = P.C + (size_t)t * P.ldc + n;
+    *c = P.accumulate ? *c + acc : acc;
+}
+
+constexpr int LM_T = 64, LM_N = 64, LM_K = 32;
+
+template <bool OPS32>
+__global__ void __launch_bounds__(256) k_lin_mfma(LinArgs P)
+{
+    // bf16 operands: [64][40] halfs per matrix (row stride 80 bytes: 16-byte aligned fragments);
+    // 32-bit operands: [64][33] floats per matrix
+    __shared__ __attribute__((aligned(16))) char smem[OPS32 ? 2 * LM_T * 33 * 4 : 2 * LM_T * 40 * 2];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int i = lane & 31, g = lane >> 5;
+    const int wm = wave & 1, wn = wave >> 1;
+    const int t0 = blockIdx.y * LM_T, n0 = blockIdx.x * LM_N;
+    const int lr = tid >> 2, lc = (tid & 3) * 8;      // this thread stages 8 consecutive k of row lr
+    f32x16v acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+
+    for (int k0 = 0; k0 < P.K; k0 += LM_K) {
+        float a8[8], w8[8];
+        {
+            const int t = t0 + lr, n = n0 + lr, k = k0 + lc;
+            const bool in_a = t < P.T, in_w = n < P.N;
+            if (P.vec && k + 8 <= P.K) {
+                if (in_a) {
+                    const float4 v0 = *reinterpret_cast<const float4 *>(P.A + (size_t)t * P.lda + k);
+                    const float4 v1 = *reinterpret_cast<const float4 *>(P.A + (size_t)t * P.lda + k + 4);
+                    a8[0] = v0.x; a8[1] = v0.y; a8[2] = v0.z; a8[3] = v0.w; a8[4] = v1.x; a8[5] = v1.y; a8[6] = v1.z; a8[7] = v1.w;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) a8[e] = 0.0f;
+                }
+                if (in_w) {
+                    const u32x4v wv = *reinterpret_cast<const u32x4v *>(P.W + (size_t)n * P.K + k);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) { w8[2 * e] = __uint_as_float(wv[e] << 16); w8[2 * e + 1] = __uint_as_float(wv[e] & 0xFFFF0000u); }
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) w8[e] = 0.0f;
+                }
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const bool kin = k + e < P.K;
+                    a8[e] = in_a && kin ? P.A[(size_t)t * P.lda + k + e] : 0.0f;
+                    w8[e] = in_w && kin ? bf2f(P.W[(size_t)n * P.K + k + e]) : 0.0f;
+                }
+            }
+        }
+        __syncthreads();      // the previous step's fragments have been read
+        if constexpr (OPS32) {
+            float *As = reinterpret_cast<float *>(smem), *Ws = As + LM_T * 33;
+#pragma unroll
+            for (int e = 0; e < 8; e++) { As[lr * 33 + lc + e] = a8[e]; Ws[lr * 33 + lc + e] = w8[e]; }
+        } else {
+            bf16_t *As = reinterpret_cast<bf16_t *>(smem), *Ws = As + LM_T * 40;
+            u32x4v av, wv;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                av[e] = (uint32_t)f2bf(a8[2 * e]) | ((uint32_t)f2bf(a8[2 * e + 1]) << 16);
+                wv[e] = (__float_as_uint(w8[2 * e]) >> 16) | (__float_as_uint(w8[2 * e + 1]) & 0xFFFF0000u);
+            }
+            *reinterpret_cast<u32x4v *>(As + lr * 40 + lc) = av;
+            *reinterpret_cast<u32x4v *>(Ws + lr * 40 + lc) = wv;
+        }
+        __syncthreads();
+        if constexpr (OPS32) {
+            const float *As = reinterpret_cast<const float *>(smem), *Ws = As + LM_T * 33;
+#pragma unroll
+            for (int s = 0; s < LM_K / 2; s++)
+                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(As[(32 * wm + i) * 33 + 2 * s + g], Ws[(32 * wn + i) * 33 + 2 * s + g], acc, 0, 0, 0);
+        } else {
+            const bf16_t *As = reinterpret_cast<const bf16_t *>(smem), *Ws = As + LM_T * 40;
+#pragma unroll
+            for (int s = 0; s < LM_K / 16; s++) {
+                const bf16x8v af = __builtin_bit_cast(bf16x8v, *reinterpret_cast<const u32x4v *>(As + (32 * wm + i) * 40 + 16 * s + 8 * g));
+                const bf16x8v wf = __builtin_bit_cast(bf16x8v, *reinterpret_cast<const u32x4v *>(Ws + (32 * wn + i) * 40 + 16 * s + 8 * g));
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af, wf, acc, 0, 0, 0);
+            }
+        }
+    }
+    const int n = n0 + 32 * wn + i;
+    if (n < P.N) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int t = t0 + 32 * wm + (r & 3) + 8 * (r >> 2) + 4 * g;
+            if (t < P.T) lin_store(P, t, n, acc[r]);
+        }
+    }
+}
+
+// T <= TT rows; one wave per output row at a time
+template <int TT>
+__global__ void __launch_bounds__(256) k_lin_rows(LinArgs P)
+{
+    const int lane = threadIdx.x & 63;
+    const int wave = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6), nwaves = gridDim.x * (blockDim.x >> 6);
+    for (int n = wave; n < P.N; n += nwaves) {
+        float acc[TT];
+#pragma unroll
+        for (int t = 0; t < TT; t++) acc[t] = 0.0f;
+        const bf16_t *w = P.W + (size_t)n * P.K;
+        if (P.vec) {
+            for (int k = lane * 8; k < P.K; k += 512) {
+                const u32x4v wv = *reinterpret_cast<const u32x4v *>(w + k);
+                float w8[8];
+#pragma unroll
+                for (int e = 0; e < 4; e++) { w8[2 * e] = __uint_as_float(wv[e] << 16); w8[2 * e + 1] = __uint_as_float(wv[e] & 0xFFFF0000u); }
+#pragma unroll
+                for (int t = 0; t < TT; t++) {
+                    const float *a = P.A + (size_t)min(t, P.T - 1) * P.lda + k;
+                    const float4 v0 = *reinterpret_cast<const float4 *>(a), v1 = *reinterpret_cast<const float4 *>(a + 4);
+                    float s = acc[t];
+                    s = fmaf(v0.x, w8[0], s); s = fmaf(v0.y, w8[1], s); s = fmaf(v0.z, w8[2], s); s = fmaf(v0.w, w8[3], s);
+                    s = fmaf(v1.x, w8[4], s); s = fmaf(v1.y, w8[5], s); s = fmaf(v1.z, w8[6], s); s = fmaf(v1.w, w8[7], s);
+                    acc[t] = s;
+                }
+            }
+        } else {
+            for (int k = lane; k < P.K; k += 64) {
+                const float wk = bf2f(w[k]);
+#pragma unroll
+                for (int t = 0; t < TT; t++) acc[t] = fmaf(P.A[(size_t)min(t, P.T - 1) * P.lda + k], wk, acc[t]);
+            }
+        }
+#pragma unroll
+        for (int t = 0; t < TT; t++) acc[t] = wave_sum(acc[t]);
+#pragma unroll
+        for (int t = 0; t < TT; t++)
+            if (lane == t && t < P.T) lin_store(P, t, n, acc[t]);
+    }
+}
+
+} // namespace
+
+extern "C" int ifa_linear_bf16w(const void *w_bf16, size_t rows, size_t cols, const void *a_f32, size_t lda, size_t tokens,
+                                const void *bias_bf16, const void *mul_bf16, float alpha, int accumulate, int ops32,
+                                void *c_f32, size_t ldc, ifa_stream stream)
+{
+    IFA_REQUIRE(w_bf16 && a_f32 && c_f32, "ifa_linear_bf16w: null pointer");
+    IFA_REQUIRE(rows > 0 && cols > 0 && tokens > 0 && lda >= cols && ldc >= rows, "ifa_linear_bf16w: bad shape (%zu x %zu, %zu tokens, lda %zu, ldc %zu)", rows, cols, tokens, lda, ldc);
+    IFA_REQUIRE(rows < (1u << 30) && cols < (1u << 30) && tokens < (1u << 30), "ifa_linear_bf16w: dimension too large");
+    LinArgs P;
+    P.W = (const bf16_t *)w_bf16; P.A = (const float *)a_f32; P.C = (float *)c_f32;
+    P.bias = (const bf16_t *)bias_bf16; P.mul = (const bf16_t *)mul_bf16;
+    P.T = (int)tokens; P.N = (int)rows; P.K = (int)cols; P.lda = (int)lda; P.ldc = (int)ldc;
+    P.alpha = alpha; P.accumulate = accumulate ? 1 : 0;
+    // 16-byte requests need whole 8-element pieces in every row of both operands
+    P.vec = (cols % 8 == 0 && lda % 4 == 0 && ((uintptr_t)a_f32 & 15) == 0 && ((uintptr_t)w_bf16 & 15) == 0) ? 1 : 0;
+    hipStream_t s = ifa_s(stream);
+    if (tokens <= 8) {
+        const unsigned grid = (unsigned)std::min<size_t>((rows + 3) / 4, 8192);
+        if (tokens == 1) hipLaunchKernelGGL(k_lin_rows<1>, dim3(grid), dim3(256), 0, s, P);
+        else if (tokens == 2) hipLaunchKernelGGL(k_lin_rows<2>, dim3(grid), dim3(256), 0, s, P);
+        else if (tokens <= 4) hipLaunchKernelGGL(k_lin_rows<4>, dim3(grid), dim3(256), 0, s, P);
+        else hipLaunchKernelGGL(k_lin_rows<8>, dim3(grid), dim3(256), 0, s, P);
+    } else {
+        const dim3 grid(ifa_cdiv(rows, LM_N), ifa_cdiv(tokens, LM_T));
+        if (ops32) hipLaunchKernelGGL(k_lin_mfma<true>, grid, dim3(256), 0, s, P);
+        else hipLaunchKernelGGL(k_lin_mfma<false>, grid, dim3(256), 0, s, P);
+    }
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}

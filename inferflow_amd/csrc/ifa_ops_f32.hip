@@ -1,0 +1,143 @@
+// ifa_ops_f32.hip -- element-wise and row ops on 32-bit activations with bfloat16 parameters: embedding rows with a sinusoidal
+// position vector, layer / RMS norm, gated activations, greedy argmax, and the conversions the F16 interfaces need.
+#include "ifa_host.h"
+#include "ifa_f32_common.h"
+
+using namespace ifa32;
+
+namespace {
+
+// x[t][c] = embed[token_t][c] + pe(pos_t)[c];  pe[2i] = sin(p w_i), pe[2i + 1] = cos(p w_i), w_i = base^(-2i / width).
+// The angle of position p reaches hundreds of radians where one fp32 ulp is already 1e-4: it is formed in double.
+__global__ void __launch_bounds__(256) k_embed_sinpos(const bf16_t *__restrict__ embed, int vocab, int width, const int *__restrict__ tokens,
+                                                      const int *__restrict__ positions, float base_log, float *__restrict__ x)
+{
+    const int t = blockIdx.x;
+    const int tok = min(max(tokens[t], 0), vocab - 1);
+    const double p = (double)positions[t];
+    for (int c = threadIdx.x; c < width; c += blockDim.x) {
+        const int i2 = c & ~1;
+        const double w = exp(-(double)i2 / (double)width * (double)base_log);
+        const double a = p * w;
+        const float pe = (float)((c & 1) ? cos(a) : sin(a));
+        x[(size_t)t * width + c] = bf2f(embed[(size_t)tok * width + c]) + pe;
+    }
+}
+
+// kind 0: y = x / sqrt(mean(x^2) + eps) * w;  kind 1: y = (x - mean) / sqrt(mean((x - mean)^2) + eps) * w.  w may be null.
+__global__ void __launch_bounds__(256) k_norm_f32(int kind, const float *__restrict__ x, size_t ldx, int cols, const bf16_t *__restrict__ w, float eps,
+                                                  float *__restrict__ y, size_t ldy)
+{
+    __shared__ float red[17];
+    const float *xr = x + (size_t)blockIdx.x * ldx;
+    float *yr = y + (size_t)blockIdx.x * ldy;
+    float mean = 0.0f;
+    if (kind == 1) {
+        float s = 0.0f;
+        for (int c = threadIdx.x; c < cols; c += blockDim.x) s += xr[c];
+        mean = block_sum(s, red) / (float)cols;
+    }
+    float q = 0.0f;
+    for (int c = threadIdx.x; c < cols; c += blockDim.x) { const float d = xr[c] - mean; q += d * d; }
+    const float rinv = 1.0f / sqrtf(block_sum(q, red) / (float)cols + eps);
+    for (int c = threadIdx.x; c < cols; c += blockDim.x) {
+        const float v = (xr[c] - mean) * rinv;
+        yr[c] = w ? v * bf2f(w[c]) : v;
+    }
+}
+
+// out[t][c] = act(gu[t][c]) * gu[t][F + c]
+__global__ void __launch_bounds__(256) k_glu_f32(int kind, const float *__restrict__ gu, size_t ld, int F, float *__restrict__ out, size_t ldo)
+{
+    const float *g = gu + (size_t)blockIdx.y * ld;
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= F) return;
+    const float a = g[c], u = g[F + c];
+    const float act = kind == 0 ? silu_exact(a) : (kind == 1 ? gelu_tanh_f(a) : fmaxf(a, 0.0f));
+    out[(size_t)blockIdx.y * ldo + c] = act * u;
+}
+
+__global__ void __launch_bounds__(256) k_argmax_f32(const float *__restrict__ logits, int n, size_t row_stride, const int *__restrict__ excluded,
+                                                    int *__restrict__ out)
+{
+    __shared__ float bv[4]; __shared__ int bi[4];
+    const float *r = logits + (size_t)blockIdx.x * row_stride;
+    int ex[3] = {-1, -1, -1};
+    if (excluded) { const int ne = min(excluded[0], 3); for (int e = 0; e < ne; e++) ex[e] = excluded[1 + e]; }
+    float best = -INFINITY; int idx = 0x7FFFFFFF;
+    for (int c = threadIdx.x; c < n; c += blockDim.x) {
+        if (c == ex[0] || c == ex[1] || c == ex[2]) continue;
+        const float v = r[c];
+        if (v > best || (v == best && c < idx)) { best = v; idx = c; }
+    }
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, 64); const int oi = __shfl_xor(idx, o, 64);
+        if (ov > best || (ov == best && oi < idx)) { best = ov; idx = oi; }
+    }
+    if ((threadIdx.x & 63) == 0) { bv[threadIdx.x >> 6] = best; bi[threadIdx.x >> 6] = idx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 4; w++) if (bv[w] > best || (bv[w] == best && bi[w] < idx)) { best = bv[w]; idx = bi[w]; }
+        out[blockIdx.x] = idx == 0x7FFFFFFF ? 0 : idx;
+    }
+}
+
+__global__ void __launch_bounds__(256) k_f32_to_f16(const float *__restrict__ src, size_t n, _Float16 *__restrict__ dst)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) dst[i] = (_Float16)src[i];
+}
+
+} // namespace
+
+extern "C" {
+
+int ifa_embed_sinpos_f32(const void *embed_bf16, int vocab, int width, const int *tokens_dev, const int *positions_dev, size_t tokens,
+                         float base, void *x_f32, ifa_stream stream)
+{
+    IFA_REQUIRE(embed_bf16 && tokens_dev && positions_dev && x_f32, "ifa_embed_sinpos_f32: null pointer");
+    IFA_REQUIRE(vocab > 0 && width > 0 && tokens > 0 && base > 1.0f, "ifa_embed_sinpos_f32: bad shape");
+    hipLaunchKernelGGL(k_embed_sinpos, dim3((unsigned)tokens), dim3(256), 0, ifa_s(stream), (const bf16_t *)embed_bf16, vocab, width, tokens_dev,
+                       positions_dev, logf(base), (float *)x_f32);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_layernorm_f32(int kind, const void *x_f32, size_t ldx, size_t rows, size_t cols, const void *w_bf16, float eps, void *y_f32, size_t ldy,
+                      ifa_stream stream)
+{
+    IFA_REQUIRE(x_f32 && y_f32, "ifa_layernorm_f32: null pointer");
+    IFA_REQUIRE((kind == 0 || kind == 1) && rows > 0 && cols > 0 && ldx >= cols && ldy >= cols, "ifa_layernorm_f32: bad arguments");
+    hipLaunchKernelGGL(k_norm_f32, dim3((unsigned)rows), dim3(256), 0, ifa_s(stream), kind, (const float *)x_f32, ldx, (int)cols,
+                       (const bf16_t *)w_bf16, eps, (float *)y_f32, ldy);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_glu_f32(int kind, const void *gate_up_f32, size_t ld, size_t rows, size_t cols, void *out_f32, size_t ldo, ifa_stream stream)
+{
+    IFA_REQUIRE(gate_up_f32 && out_f32, "ifa_glu_f32: null pointer");
+    IFA_REQUIRE(kind >= 0 && kind <= 2 && rows > 0 && cols > 0 && ld >= 2 * cols && ldo >= cols, "ifa_glu_f32: bad arguments");
+    hipLaunchKernelGGL(k_glu_f32, dim3(ifa_cdiv(cols, 256), (unsigned)rows), dim3(256), 0, ifa_s(stream), kind, (const float *)gate_up_f32, ld,
+                       (int)cols, (float *)out_f32, ldo);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_argmax_rows_f32(const void *logits_f32, size_t n, size_t row_stride, size_t rows, const int *excluded_dev, int *out_dev, ifa_stream stream)
+{
+    IFA_REQUIRE(logits_f32 && out_dev && n > 0 && rows > 0 && n < (1u << 30), "ifa_argmax_rows_f32: bad arguments");
+    hipLaunchKernelGGL(k_argmax_f32, dim3((unsigned)rows), dim3(256), 0, ifa_s(stream), (const float *)logits_f32, (int)n, row_stride, excluded_dev, out_dev);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_convert_f32_f16(const void *src_f32, size_t n, void *dst_f16, ifa_stream stream)
+{
+    IFA_REQUIRE(src_f32 && dst_f16 && n > 0, "ifa_convert_f32_f16: bad arguments");
+    hipLaunchKernelGGL(k_f32_to_f16, dim3(ifa_cdiv(n, 256)), dim3(256), 0, ifa_s(stream), (const float *)src_f32, n, (_Float16 *)dst_f16);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+} // extern "C"

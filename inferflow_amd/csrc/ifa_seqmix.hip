@@ -1,0 +1,269 @@
+// ifa_seqmix.hip -- sequence mixers with a recurrent state instead of a key / value cache, on 32-bit activations:
+//   * short causal convolution per channel + SiLU (+ unit-norm of head groups), its tail carried per sequence
+//   * per-head matrix state S [dk][dv] advanced token by token:
+//       kind 0  linear attention with a constant decay per head:  S <- d S + k v^T;                      o = S^T q
+//     (in_act = 1: q, k, v pass SiLU as they are read)
+//       kind 1  gated delta rule:                                 S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
+//   * the gates of the delta rule (beta = sigmoid, g = exp(-exp(A_log) softplus(a + dt_bias)))
+//   * RMS norm over channel groups with a weight and an output gate (sigmoid or SiLU)
+// Everything that enters a recurrence is fp32; states live in fp32 in the slot arena of the worker (a table of one
+// base pointer per slot + an offset per layer).  A sequence that starts at position 0 starts from a zero state,
+// whatever the slot held before.
+#include "ifa_host.h"
+#include "ifa_f32_common.h"
+
+using namespace ifa32;
+
+namespace {
+
+// grid: one workgroup per row.  y[t][c] = silu(sum_j w[c][j] in(i - (taps - 1) + j)[c]); in(idx) for idx < 0 comes from the
+// sequence's carried tail (rows [taps - 1][C], oldest first) or is zero at the start of a sequence.  Then channels
+// [0, norm_cols) are turned into unit vectors in groups of gdim (x / sqrt(sum x^2 + l2_eps)) and channels [0, scale_cols)
+// are multiplied by qscale.
+__global__ void __launch_bounds__(256) k_shortconv_silu(const float *__restrict__ x, size_t ldx, int C, int taps, const bf16_t *__restrict__ w,
+                                                        const SeqDesc *__restrict__ seqs, const int *__restrict__ row_seq,
+                                                        float *const *__restrict__ slot_base, size_t state_off, int norm_cols, int gdim,
+                                                        float l2_eps, int scale_cols, float qscale, float *__restrict__ y, size_t ldy)
+{
+    extern __shared__ float ys[];
+    const int t = blockIdx.x;
+    const SeqDesc sd = seqs[row_seq[t]];
+    const int i = t - sd.row0;
+    const float *tail = sd.pos0 > 0 ? slot_base[sd.slot] + state_off : nullptr;
+    for (int c = threadIdx.x; c < C; c += blockDim.x) {
+        float acc = 0.0f;
+        for (int j = 0; j < taps; j++) {
+            const int idx = i - (taps - 1) + j;
+            float v;
+            if (idx >= 0) v = x[(size_t)(sd.row0 + idx) * ldx + c];
+            else v = tail ? tail[(size_t)(taps - 1 + idx) * C + c] : 0.0f;
+            acc = fmaf(bf2f(w[(size_t)c * taps + j]), v, acc);
+        }
+        ys[c] = silu_exact(acc);
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int ngroups = gdim > 0 ? norm_cols / gdim : 0;
+    for (int gidx = wave; gidx < ngroups; gidx += nw) {
+        float s = 0.0f;
+        for (int e = lane; e < gdim; e += 64) { const float v = ys[gidx * gdim + e]; s = fmaf(v, v, s); }
+        s = wave_sum(s);
+        const float r = 1.0f / sqrtf(s + l2_eps);
+        for (int e = lane; e < gdim; e += 64) ys[gidx * gdim + e] *= r;
+    }
+    __syncthreads();
+    for (int c = threadIdx.x; c < C; c += blockDim.x) y[(size_t)t * ldy + c] = c < scale_cols ? ys[c] * qscale : ys[c];
+}
+
+// grid: one workgroup per sequence.  The carried tail becomes the last taps - 1 inputs of (old tail, this step's rows).
+__global__ void __launch_bounds__(256) k_shortconv_tail(const float *__restrict__ x, size_t ldx, int C, int taps, const SeqDesc *__restrict__ seqs,
+                                                        float *const *__restrict__ slot_base, size_t state_off)
+{
+    const SeqDesc sd = seqs[blockIdx.x];
+    float *tail = slot_base[sd.slot] + state_off;
+    const int keep = taps - 1;
+    for (int c = threadIdx.x; c < C; c += blockDim.x)
+        for (int r = 0; r < keep; r++) {          // ascending r: a value read from the old tail lies above what was written so far
+            const int idx = sd.n - keep + r;      // index into this step's rows
+            float v;
+            if (idx >= 0) v = x[(size_t)(sd.row0 + idx) * ldx + c];
+            else v = sd.pos0 > 0 ? tail[(size_t)(keep + idx) * C + c] : 0.0f;
+            tail[(size_t)r * C + c] = v;
+        }
+}
+
+// beta[t][h] = sigmoid(b[t][h]);  g[t][h] = exp(-exp(A_log[h]) * softplus(a[t][h] + dt_bias[h]))
+__global__ void __launch_bounds__(256) k_delta_gates(const float *__restrict__ b, size_t ldb, const float *__restrict__ a, size_t lda, int H, int T,
+                                                     const bf16_t *__restrict__ A_log, const bf16_t *__restrict__ dt_bias, float *__restrict__ beta,
+                                                     float *__restrict__ g)
+{
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= T * H) return;
+    const int t = idx / H, h = idx % H;
+    beta[idx] = sigmoid_f(b[(size_t)t * ldb + h]);
+    g[idx] = expf(-expf(bf2f(A_log[h])) * softplus_f(a[(size_t)t * lda + h] + bf2f(dt_bias[h])));
+}
+
+struct ScanArgs {
+    const float *q, *k, *v; size_t ldq, ldk, ldv;
+    int heads, qk_heads, dk, dv, in_act;
+    const float *decay_head, *decay_row, *beta_row;
+    const SeqDesc *seqs; float *const *slot_base; size_t state_off;
+    float *out; size_t ldo;
+};
+
+constexpr int SCAN_DKL = 4;       // dk <= 64 * SCAN_DKL
+
+// grid (sequences * heads, ceil(dv / 64)), one wave per workgroup: the columns of S are independent in both recurrences, so
+// each lane owns one column S[:, j] (in LDS, [dk][64]: conflict-free) and needs q_t, k_t (broadcast from LDS) and its v_t[j].
+// The next token's operands are requested before the current token is computed.
+template <int KIND>
+__global__ void __launch_bounds__(64) k_state_scan(ScanArgs P)
+{
+    extern __shared__ float sm[];
+    float *S = sm, *qs = sm + (size_t)P.dk * 64, *ks = qs + P.dk;
+    const int seq = blockIdx.x / P.heads, h = blockIdx.x % P.heads;
+    const int lane = threadIdx.x, j = blockIdx.y * 64 + lane;
+    const bool live = j < P.dv;
+    const int jc = live ? j : P.dv - 1;
+    const int qh = h / (P.heads / P.qk_heads);
+    const SeqDesc sd = P.seqs[seq];
+    float *state = P.slot_base[sd.slot] + P.state_off + (size_t)h * P.dk * P.dv;
+    const int dk = P.dk;
+    if (sd.pos0 > 0) for (int i = 0; i < dk; i++) S[i * 64 + lane] = state[(size_t)i * P.dv + jc];
+    else for (int i = 0; i < dk; i++) S[i * 64 + lane] = 0.0f;
+    const float dconst = KIND == 0 ? P.decay_head[h] : 0.0f;
+    float qr[SCAN_DKL], kr[SCAN_DKL], vr, gr = 0.0f, br = 0.0f;
+    auto request = [&](int t) {
+        const size_t row = (size_t)(sd.row0 + t);
+#pragma unroll
+        for (int e = 0; e < SCAN_DKL; e++) {
+            const int i = lane + 64 * e;
+            if (i < dk) {
+                qr[e] = P.q[row * P.ldq + (size_t)qh * dk + i]; kr[e] = P.k[row * P.ldk + (size_t)qh * dk + i];
+                if (P.in_act) { qr[e] = silu_exact(qr[e]); kr[e] = silu_exact(kr[e]); }
+            }
+        }
+        vr = P.v[row * P.ldv + (size_t)h * P.dv + jc];
+        if (P.in_act) vr = silu_exact(vr);
+        if (KIND == 1) { gr = P.decay_row[row * P.heads + h]; br = P.beta_row[row * P.heads + h]; }
+    };
+    if (sd.n > 0) request(0);
+    for (int t = 0; t < sd.n; t++) {
+        __syncthreads();          // the previous token's reads of qs / ks are done
+#pragma unroll
+        for (int e = 0; e < SCAN_DKL; e++) { const int i = lane + 64 * e; if (i < dk) { qs[i] = qr[e]; ks[i] = kr[e]; } }
+        const float vt = vr, gt = gr, bt = br;
+        __syncthreads();
+        if (t + 1 < sd.n) request(t + 1);
+        float o = 0.0f;
+        if (KIND == 0) {
+            for (int i = 0; i < dk; i++) {
+                const float s = fmaf(dconst, S[i * 64 + lane], ks[i] * vt);
+                S[i * 64 + lane] = s;
+                o = fmaf(s, qs[i], o);
+            }
+        } else {
+            float r = 0.0f;
+            for (int i = 0; i < dk; i++) {
+                const float s = gt * S[i * 64 + lane];
+                S[i * 64 + lane] = s;
+                r = fmaf(s, ks[i], r);
+            }
+            const float u = bt * (vt - r);
+            for (int i = 0; i < dk; i++) {
+                const float s = fmaf(ks[i], u, S[i * 64 + lane]);
+                S[i * 64 + lane] = s;
+                o = fmaf(s, qs[i], o);
+            }
+        }
+        if (live) P.out[(size_t)(sd.row0 + t) * P.ldo + (size_t)h * P.dv + j] = o;
+    }
+    if (live) for (int i = 0; i < dk; i++) state[(size_t)i * P.dv + j] = S[i * 64 + lane];
+}
+
+// y[t][c] = o[t][c] / sqrt(mean_group(o^2) + eps) * w[c % wlen] * act(gate[t][c]); one workgroup per row, a wave per group
+__global__ void __launch_bounds__(256) k_gated_groupnorm(const float *__restrict__ o, size_t ldo, int C, int group, const bf16_t *__restrict__ w, int wlen,
+                                                         const float *__restrict__ gate, size_t ldg, int gate_act, float eps, float *__restrict__ y,
+                                                         size_t ldy)
+{
+    const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const float *orow = o + (size_t)t * ldo, *grow = gate + (size_t)t * ldg;
+    float *yrow = y + (size_t)t * ldy;
+    for (int gi = wave; gi < C / group; gi += nw) {
+        float s = 0.0f;
+        for (int e = lane; e < group; e += 64) { const float v = orow[gi * group + e]; s = fmaf(v, v, s); }
+        s = wave_sum(s);
+        const float r = 1.0f / sqrtf(s / (float)group + eps);
+        for (int e = lane; e < group; e += 64) {
+            const int c = gi * group + e;
+            const float gv = grow[c];
+            const float ga = gate_act == 0 ? sigmoid_f(gv) : silu_exact(gv);
+            yrow[c] = orow[c] * r * bf2f(w[c % wlen]) * ga;
+        }
+    }
+}
+
+} // namespace
+
+extern "C" {
+
+int ifa_shortconv_silu_f32(const void *x_f32, size_t ldx, int channels, int taps, const void *w_bf16, const void *seqs_dev, const int *row_seq_dev,
+                           size_t rows, void *const *slot_base_dev, size_t state_off, int norm_cols, int group_dim, float l2_eps, int scale_cols,
+                           float scale, void *y_f32, size_t ldy, ifa_stream stream)
+{
+    IFA_REQUIRE(x_f32 && w_bf16 && seqs_dev && row_seq_dev && slot_base_dev && y_f32, "ifa_shortconv_silu_f32: null pointer");
+    IFA_REQUIRE(channels > 0 && taps >= 1 && taps <= 64 && rows > 0 && ldx >= (size_t)channels && ldy >= (size_t)channels, "ifa_shortconv_silu_f32: bad shape");
+    IFA_REQUIRE(norm_cols >= 0 && norm_cols <= channels && scale_cols >= 0 && scale_cols <= channels && (norm_cols == 0 || (group_dim > 0 && norm_cols % group_dim == 0)),
+                "ifa_shortconv_silu_f32: bad norm groups");
+    IFA_REQUIRE((size_t)channels * 4 <= 64 * 1024, "ifa_shortconv_silu_f32: %d channels do not fit the LDS row", channels);
+    hipLaunchKernelGGL(k_shortconv_silu, dim3((unsigned)rows), dim3(256), (size_t)channels * 4, ifa_s(stream), (const float *)x_f32, ldx, channels, taps,
+                       (const bf16_t *)w_bf16, (const SeqDesc *)seqs_dev, row_seq_dev, (float *const *)slot_base_dev, state_off, norm_cols, group_dim, l2_eps,
+                       scale_cols, scale, (float *)y_f32, ldy);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_shortconv_tail_f32(const void *x_f32, size_t ldx, int channels, int taps, const void *seqs_dev, int n_seqs, void *const *slot_base_dev,
+                           size_t state_off, ifa_stream stream)
+{
+    IFA_REQUIRE(x_f32 && seqs_dev && slot_base_dev, "ifa_shortconv_tail_f32: null pointer");
+    IFA_REQUIRE(channels > 0 && taps >= 1 && n_seqs > 0 && ldx >= (size_t)channels, "ifa_shortconv_tail_f32: bad shape");
+    if (taps == 1) return IFA_OK;
+    hipLaunchKernelGGL(k_shortconv_tail, dim3((unsigned)n_seqs), dim3(256), 0, ifa_s(stream), (const float *)x_f32, ldx, channels, taps,
+                       (const SeqDesc *)seqs_dev, (float *const *)slot_base_dev, state_off);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_delta_gates_f32(const void *b_f32, size_t ldb, const void *a_f32, size_t lda, int heads, size_t rows, const void *a_log_bf16,
+                        const void *dt_bias_bf16, void *beta_f32, void *decay_f32, ifa_stream stream)
+{
+    IFA_REQUIRE(b_f32 && a_f32 && a_log_bf16 && dt_bias_bf16 && beta_f32 && decay_f32, "ifa_delta_gates_f32: null pointer");
+    IFA_REQUIRE(heads > 0 && rows > 0 && ldb >= (size_t)heads && lda >= (size_t)heads, "ifa_delta_gates_f32: bad shape");
+    hipLaunchKernelGGL(k_delta_gates, dim3(ifa_cdiv(rows * heads, 256)), dim3(256), 0, ifa_s(stream), (const float *)b_f32, ldb, (const float *)a_f32, lda,
+                       heads, (int)rows, (const bf16_t *)a_log_bf16, (const bf16_t *)dt_bias_bf16, (float *)beta_f32, (float *)decay_f32);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_state_scan_f32(int kind, int in_act, const void *q_f32, size_t ldq, const void *k_f32, size_t ldk, const void *v_f32, size_t ldv, int heads, int qk_heads,
+                       int dk, int dv, const void *decay_head_f32, const void *decay_row_f32, const void *beta_row_f32, const void *seqs_dev, int n_seqs,
+                       void *const *slot_base_dev, size_t state_off, void *out_f32, size_t ldo, ifa_stream stream)
+{
+    IFA_REQUIRE(q_f32 && k_f32 && v_f32 && seqs_dev && slot_base_dev && out_f32, "ifa_state_scan_f32: null pointer");
+    IFA_REQUIRE(kind == 0 || kind == 1, "ifa_state_scan_f32: kind %d", kind);
+    IFA_REQUIRE(heads > 0 && qk_heads > 0 && heads % qk_heads == 0 && dk > 0 && dv > 0 && n_seqs > 0, "ifa_state_scan_f32: bad shape");
+    IFA_REQUIRE(dk <= 64 * SCAN_DKL, "ifa_state_scan_f32: key size %d above %d", dk, 64 * SCAN_DKL);
+    IFA_REQUIRE(kind == 0 ? decay_head_f32 != nullptr : (decay_row_f32 && beta_row_f32), "ifa_state_scan_f32: the gates of kind %d are missing", kind);
+    ScanArgs P;
+    P.q = (const float *)q_f32; P.k = (const float *)k_f32; P.v = (const float *)v_f32; P.ldq = ldq; P.ldk = ldk; P.ldv = ldv;
+    P.heads = heads; P.qk_heads = qk_heads; P.dk = dk; P.dv = dv; P.in_act = in_act ? 1 : 0;
+    P.decay_head = (const float *)decay_head_f32; P.decay_row = (const float *)decay_row_f32; P.beta_row = (const float *)beta_row_f32;
+    P.seqs = (const SeqDesc *)seqs_dev; P.slot_base = (float *const *)slot_base_dev; P.state_off = state_off;
+    P.out = (float *)out_f32; P.ldo = ldo;
+    const size_t smem = ((size_t)dk * 64 + 2 * (size_t)dk) * 4;
+    const dim3 grid((unsigned)(n_seqs * heads), ifa_cdiv((size_t)dv, 64));
+    if (kind == 0) {
+        IFA_HIP_CHECK(hipFuncSetAttribute((const void *)k_state_scan<0>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        hipLaunchKernelGGL(k_state_scan<0>, grid, dim3(64), smem, ifa_s(stream), P);
+    } else {
+        IFA_HIP_CHECK(hipFuncSetAttribute((const void *)k_state_scan<1>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+        hipLaunchKernelGGL(k_state_scan<1>, grid, dim3(64), smem, ifa_s(stream), P);
+    }
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_gated_groupnorm_f32(const void *o_f32, size_t ldo, size_t rows, int channels, int group, const void *w_bf16, int wlen, const void *gate_f32,
+                            size_t ldg, int gate_act, float eps, void *y_f32, size_t ldy, ifa_stream stream)
+{
+    IFA_REQUIRE(o_f32 && w_bf16 && gate_f32 && y_f32, "ifa_gated_groupnorm_f32: null pointer");
+    IFA_REQUIRE(rows > 0 && channels > 0 && group > 0 && channels % group == 0 && wlen > 0 && (gate_act == 0 || gate_act == 1), "ifa_gated_groupnorm_f32: bad arguments");
+    hipLaunchKernelGGL(k_gated_groupnorm, dim3((unsigned)rows), dim3(256), 0, ifa_s(stream), (const float *)o_f32, ldo, channels, group,
+                       (const bf16_t *)w_bf16, wlen, (const float *)gate_f32, ldg, gate_act, eps, (float *)y_f32, ldy);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+} // extern "C"

@@ -33,6 +33,18 @@ ifa_engine *ifa_engine_create(const char *ini_path, const char *section, const c
     return e;
 }
 
+ifa_engine *ifa_engine_create_from_dir(const char *model_dir, const char *compute_dtype, int max_context_len, int max_concurrent_queries,
+                                       int return_output_tensors)
+{
+    if (!model_dir) { EngineSetError("ifa_engine_create_from_dir: null argument"); return nullptr; }
+    InferenceConfig cfg;
+    if (!InferenceEngine::LoadConfigForModelDir(cfg, model_dir, compute_dtype ? compute_dtype : "", max_context_len, max_concurrent_queries)) return nullptr;
+    cfg.return_output_tensors_f32 = return_output_tensors != 0;
+    ifa_engine *e = new ifa_engine();
+    if (!e->engine.Init(cfg)) { delete e; return nullptr; }
+    return e;
+}
+
 void ifa_engine_destroy(ifa_engine *e) { delete e; }
 
 int ifa_engine_add_query(ifa_engine *e, const int *tokens, int n_tokens)
@@ -161,6 +173,17 @@ int ifa_engine_last_logits(ifa_engine *e, int query_id, uint16_t *dst_f16, size_
     if (rows) *rows = it->second.output_rows;
     if (cols) *cols = it->second.output_cols;
     if (dst_f16) memcpy(dst_f16, it->second.output_tensor.data(), std::min(capacity, it->second.output_tensor.size()) * 2);
+    return 1;
+}
+
+int ifa_engine_last_logits_f32(ifa_engine *e, int query_id, float *dst_f32, size_t capacity, int *rows, int *cols)
+{
+    if (!e) return 0;
+    auto it = e->last.find(query_id);
+    if (it == e->last.end()) { EngineSetError("no result for query %d", query_id); return 0; }
+    if (rows) *rows = it->second.output_rows;
+    if (cols) *cols = it->second.output_cols;
+    if (dst_f32) memcpy(dst_f32, it->second.output_tensor_f32.data(), std::min(capacity, it->second.output_tensor_f32.size()) * 4);
     return 1;
 }
 

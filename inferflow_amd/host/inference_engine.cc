@@ -155,7 +155,18 @@ static bool LoadModelSpec(ModelSpec &spec, const IniConfig &cfg, const std::stri
     }
     if (spec.dir.back() != '/' && spec.dir.back() != '\\') spec.dir += '/';
     if (!cfg.GetItem(section, "model_specification_file", spec.spec_file)) cfg.GetItem(section, "model_spec_file", spec.spec_file);
-    if (spec.spec_file.empty()) { EngineSetError("The specification file of model \"%s\" should not be empty", spec.sid.c_str()); return false; }
+    // a directory whose config.json names a registered layer-list architecture needs no specification file
+    std::string arch;
+    const bool layered = spec.spec_file.empty() && LayeredArchitectureOf(spec.dir, arch);
+    if (spec.spec_file.empty() && !layered) { EngineSetError("The specification file of model \"%s\" should not be empty", spec.sid.c_str()); return false; }
+    {
+        std::string cd;
+        if (cfg.GetItem(section, "compute_dtype", cd) && !cd.empty()) {
+            cd = IniConfig::Lower(cd);
+            if (cd != "float32" && cd != "f32" && cd != "bfloat16" && cd != "bf16") { EngineSetError("Invalid compute_dtype for model %s", spec.sid.c_str()); return false; }
+            spec.exact_fp32 = cd[0] == 'f';
+        }
+    }
     cfg.GetItem(section, "decoding_strategy", spec.decoding_strategy);
     cfg.GetItem(section, "decoder_input_template", spec.decoder_input_template);
     cfg.GetItem(section, "prompt_template", spec.decoder_input_template);
@@ -186,6 +197,7 @@ static bool LoadModelSpec(ModelSpec &spec, const IniConfig &cfg, const std::stri
     cfg.GetItem(section, "tensor_quant_threshold", spec.tensor_quant_threshold);
     if (!LoadDeviceGroups(spec.device_groups, cfg, section, "devices")) return false;
     cfg.GetItem(section, "max_context_len", spec.max_context_len);
+    if (layered) return LoadLayeredSpec(spec);
     const bool is_abs = !spec.spec_file.empty() && spec.spec_file[0] == '/';
     return LoadModelSpecJson(spec, is_abs ? spec.spec_file : spec.dir + spec.spec_file);
 }
@@ -226,10 +238,34 @@ bool InferenceEngine::LoadConfig(InferenceConfig &config, const std::string &con
     cfg.GetItem(section, "max_concurrent_queries", config.max_concurrent_queries);
     cfg.GetItem(section, "cpu_threads", config.cpu_threads);
     cfg.GetItem(section, "return_output_tensors", config.return_output_tensors);
+    cfg.GetItem(section, "return_output_tensors_f32", config.return_output_tensors_f32);
     cfg.GetItem(section, "dynamic_batching_min_queries", config.dynamic_batching_min_queries);
     cfg.GetItem(section, "force_partition_path", config.force_partition_path);
     cfg.GetItem(section, "is_study_mode", config.debug.is_study_mode);
     cfg.GetItem(section, "show_tensors", config.debug.show_tensors);
+    return true;
+}
+
+bool InferenceEngine::LoadConfigForModelDir(InferenceConfig &config, const std::string &model_dir, const std::string &compute_dtype, int max_context_len,
+                                            int max_concurrent_queries, int device)
+{
+    ModelSpec spec;
+    spec.dir = model_dir;
+    if (spec.dir.empty()) { EngineSetError("The model directory should not be empty"); return false; }
+    if (spec.dir.back() != '/') spec.dir += '/';
+    std::string arch;
+    if (!LayeredArchitectureOf(spec.dir, arch)) { EngineSetError("%sconfig.json names no registered architecture", spec.dir.c_str()); return false; }
+    spec.sid = arch;
+    const std::string cd = IniConfig::Lower(compute_dtype);
+    if (cd == "float32" || cd == "f32") spec.exact_fp32 = true;
+    else if (!(cd.empty() || cd == "bfloat16" || cd == "bf16")) { EngineSetError("compute dtype \"%s\" is not supported (bfloat16, float32)", compute_dtype.c_str()); return false; }
+    spec.max_context_len = max_context_len;
+    spec.device_groups.push_back({device});
+    if (!LoadLayeredSpec(spec)) return false;
+    config = InferenceConfig();
+    config.device_groups = spec.device_groups;
+    config.max_concurrent_queries = max_concurrent_queries;
+    config.models.push_back(spec);
     return true;
 }
 
@@ -515,6 +551,7 @@ bool InferenceEngine::Infer(InferenceResult &res)
 {
     res.items.clear(); res.perf_stat.time_map.clear();
     if (!model_) { EngineSetError("The engine is not initialized"); return false; }
+    if (!multi_ && ifa_model_is_layered(model_)) return InferLayered(res);
     const auto t0 = std::chrono::steady_clock::now();
     const int V = spec_.hyper_params.vocab_size;
     const int max_ctx = spec_.max_context_len > 0 ? spec_.max_context_len : ModelSpec::DEFAULT_MAX_CONTEXT_LEN;
@@ -633,6 +670,75 @@ bool InferenceEngine::Infer(InferenceResult &res)
         int keys[256]; float ms[256]; int n = 0;
         if (ifa_model_perf_stat(model_, keys, ms, 256, &n, 1) != IFA_OK) { EngineSetError("perf_stat: %s", ifa_last_error()); return false; }
         for (int i = 0; i < std::min(n, 256); i++) res.perf_stat.time_map[keys[i]] = ms[i];
+    }
+    if (config_.debug.enable_perf_stat)
+        res.perf_stat.time_map[0] = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();
+    return true;
+}
+
+// Layer-list models: every query with pending tokens -- whole prompts, portions of prompts, single tokens -- joins ONE step of the worker
+// (ifa_model_step_seqs): its rows are independent of what else the step holds, so the scheduler need not separate prefill from decoding.
+bool InferenceEngine::InferLayered(InferenceResult &res)
+{
+    const auto t0 = std::chrono::steady_clock::now();
+    const int V = spec_.hyper_params.vocab_size;
+    const int max_ctx = MaxContextLen();
+    std::vector<Query *> step;
+    for (auto &kv : queries_) {
+        Query &q = kv.second;
+        if (q.ended) continue;
+        if ((int)q.tokens.size() >= max_ctx) { q.ended = true; continue; }
+        if ((int)q.tokens.size() - q.processed > 0) step.push_back(&q);
+    }
+    if (step.empty()) return true;
+    const bool want_all = config_.return_output_tensors || config_.return_output_tensors_f32;
+    std::vector<int> toks, lens, pos0, slots, next(step.size(), -1);
+    for (Query *q : step) {
+        lens.push_back((int)q->tokens.size() - q->processed); pos0.push_back(q->processed); slots.push_back(q->kv_slot);
+        toks.insert(toks.end(), q->tokens.begin() + q->processed, q->tokens.end());
+    }
+    if (ifa_model_step_seqs(model_, (int)step.size(), toks.data(), lens.data(), pos0.data(), slots.data(), want_all ? 1 : 0, next.data()) != IFA_OK) {
+        EngineSetError("step failed: %s", ifa_last_error()); return false;
+    }
+    bool any_sampled = false;
+    for (Query *q : step) any_sampled = any_sampled || q->strategy != SamplingStrategyId::Greedy || host_greedy_;
+    std::vector<float> all;
+    size_t rows = 0, cols = 0;
+    if (want_all || any_sampled) {
+        void *lg = nullptr;
+        if (ifa_model_logits_f32(model_, &lg, &rows, &cols) != IFA_OK || !lg || (int)cols != V) { EngineSetError("logits: %s", ifa_last_error()); return false; }
+        all.resize(rows * cols);
+        if (ifa_memcpy_d2h(all.data(), lg, all.size() * 4, ifa_model_stream(model_)) != IFA_OK || ifa_stream_sync(ifa_model_stream(model_)) != IFA_OK) {
+            EngineSetError("logits copy: %s", ifa_last_error()); return false;
+        }
+    }
+    size_t r0 = 0;
+    for (size_t i = 0; i < step.size(); i++) {
+        Query &q = *step[i];
+        const size_t n_new = (size_t)lens[i];
+        // rows of this query in `all`: every token's (want_all or a step of single tokens) or only its last one
+        const bool per_token = rows == toks.size();
+        const size_t first = per_token ? r0 : i, count = per_token ? n_new : 1;
+        QueryInferenceResult item; item.query_id = q.id; item.prefix_len = q.processed;
+        if (want_all) {
+            item.output_rows = (int)count; item.output_cols = V;
+            if (config_.return_output_tensors_f32) item.output_tensor_f32.assign(all.begin() + first * V, all.begin() + (first + count) * V);
+            if (config_.return_output_tensors) {
+                item.output_tensor.resize(count * (size_t)V);
+                for (size_t e = 0; e < count * (size_t)V; e++) item.output_tensor[e] = FloatToHalfBits(all[first * V + e]);
+            }
+        }
+        IdWeight w; w.id = next[i]; w.weight = 1.0f;
+        item.next_tokens.push_back(w);
+        if (q.strategy != SamplingStrategyId::Greedy || host_greedy_) {
+            std::vector<uint16_t> row((size_t)V);
+            const float *src = all.data() + (first + count - 1) * V;
+            for (int e = 0; e < V; e++) row[(size_t)e] = FloatToHalfBits(src[e]);
+            if (!SampleRow(q, row.data(), item)) return false;
+        }
+        q.processed = (int)q.tokens.size();
+        r0 += n_new;
+        res.items.push_back(std::move(item));
     }
     if (config_.debug.enable_perf_stat)
         res.perf_stat.time_map[0] = std::chrono::duration<float, std::milli>(std::chrono::steady_clock::now() - t0).count();

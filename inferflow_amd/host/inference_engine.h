@@ -46,6 +46,10 @@ struct ModelSpec {
     std::vector<std::string> model_files;
     std::string model_file_format;          // "llama2.c" | "safetensors" | "synthetic"
     std::string network_structure = "transformer.llama";
+    // models described layer by layer in their own config.json (layered_model.cc): the registered architecture name; model_file_format
+    // "layered", network_structure "layered.<architecture>".  exact_fp32: matrix products keep fp32 operands (compute_dtype = float32)
+    std::string architecture;
+    bool exact_fp32 = false;
     TensorNormAlg norm_alg = TensorNormAlg::STD;
     ActivationFn activation_fn = ActivationFn::SILU;
     PositionEmbeddingAlg pos_embedding_alg = PositionEmbeddingAlg::ROPE;
@@ -88,6 +92,8 @@ struct InferenceConfig {
     int encoder_cpu_layer_count = 0, decoder_cpu_layer_count = 0, cpu_threads = 8;
     std::map<std::string, std::string> prompt_templates;
     bool return_output_tensors = false;
+    // extension: the logits of a step also as 32-bit floats (QueryInferenceResult::output_tensor_f32) from workers that compute them so
+    bool return_output_tensors_f32 = false;
     // extension: queries advancing by one token share ONE batched step (rows GEMM on the matrix cores, five launches per
     // layer) from this many on; below it each runs the fused single-query decode (Llama-2-7B Q4: 2 queries batched give
     // 825 aggregate tok/s against 690 for one after the other)
@@ -111,6 +117,7 @@ struct QueryInferenceResult {
     int prefix_len = 0;
     std::vector<IdWeight> next_tokens;          // [0] = the chosen token (greedy: weight 1; sampled: its pool probability)
     std::vector<uint16_t> output_tensor;        // F16 logits [output_rows][output_cols] if return_output_tensors
+    std::vector<float> output_tensor_f32;       // the same rows in fp32 if return_output_tensors_f32 (layer-list models)
     int output_rows = 0, output_cols = 0;
 };
 
@@ -153,6 +160,10 @@ public:
 
     static bool LoadConfig(InferenceConfig &config, const std::string &config_path,
                            const std::string &section, const std::string &data_root_dir = "");
+    // configuration for a bare model directory (config.json with a registered "architecture" + model.safetensors), no .ini:
+    // compute_dtype "bfloat16" | "float32", context length and number of concurrent queries as given
+    static bool LoadConfigForModelDir(InferenceConfig &config, const std::string &model_dir, const std::string &compute_dtype, int max_context_len,
+                                      int max_concurrent_queries, int device = 0);
     bool Init(const InferenceConfig &cfg);
 
     // > 0: query id, 0: busy (max_concurrent_queries reached), < 0: error
@@ -207,6 +218,7 @@ private:
         SamplingState sampling_state;   // Mirostat's mu, the FSD n-gram model, the EOS bypass count
     };
     bool SampleRow(Query &q, const uint16_t *logits_row, QueryInferenceResult &item);
+    bool InferLayered(InferenceResult &res);      // one step for ALL pending queries of a layer-list model, prompts and single tokens mixed
     // ---- multi-GPU partitions (devices = 0&1 | 0;1 | 0&1;2&3): one worker and one host thread per GPU, like the
     // reference's Infer_TensorParallelism / Infer_Std over GpuInferenceWorker threads (inference_engine.cc:1161-1296)
     struct MultiGpu;
@@ -235,6 +247,13 @@ const char *EngineLastError();
 void EngineSetError(const char *fmt, ...) __attribute__((format(printf, 1, 2)));
 
 // model loading (model_loader.cc)
+struct StTensorEntry { std::string file; std::string dtype; std::vector<size_t> shape; size_t begin = 0, end = 0, data_off = 0; };
+uint16_t FloatToHalfBits(float f);
+// layer-list models (layered_model.cc): is <dir>config.json one of a registered architecture; spec from it; the worker from it
+bool LayeredArchitectureOf(const std::string &dir, std::string &arch);
+bool LoadLayeredSpec(ModelSpec &spec);
+struct WorkerPlan;
+bool LoadLayered(std::vector<WorkerPlan> &plans, ModelSpec &spec);
 bool LoadModelSpecJson(ModelSpec &spec, const std::string &path);
 bool BuildWorker(ifa_model **out, ModelSpec &spec, int device);
 

@@ -1,0 +1,238 @@
+// layered_model.cc -- models described layer by layer in their own config.json ("architecture": <name>, "layers": [...]),
+// served by the layer-list worker (ifa_model_create_layered).  The registry below maps an architecture name to the reader of
+// its configuration and to its tensor names; a model directory holds config.json + model.safetensors (bfloat16 weights).
+//
+// Gelarax: width / vocab / norm.eps; every layer has one layer norm (no bias) feeding its mixer and its GELU-gated
+// feed-forward in parallel, layer scales ls1 / ls2, and a mixer of type
+//   "parallel"  windowed softmax attention with kept first tokens, soft cap, distance-bucket bias and sink ("left") beside
+//               decayed linear attention ("right"), summed with left_scale / right_scale
+//   "delta"     gated delta rule behind short causal convolutions
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <fstream>
+#include <sstream>
+
+#include "inferflow_amd.h"
+#include "inference_engine.h"
+#include "ifa_json.h"
+
+namespace inferflow_amd {
+
+bool IndexSafetensorsFile(const std::string &path, std::map<std::string, StTensorEntry> &index);      // model_loader.cc
+
+namespace {
+
+bool ReadText(const std::string &path, std::string &out)
+{
+    std::ifstream f(path, std::ios::binary);
+    if (!f) return false;
+    std::stringstream ss; ss << f.rdbuf();
+    out = ss.str();
+    return true;
+}
+
+struct LayeredDesc {
+    ifa_layered_config cfg;
+    std::vector<ifa_layer_spec> layers;
+    std::vector<std::vector<float>> decays;        // per layer: decay per linear-attention head
+};
+
+template <typename T> bool Need(const JsonValue &o, const char *key, T &out, const char *where)
+{
+    if (o.GetNumber(key, out)) return true;
+    EngineSetError("config.json: %s.%s is missing", where, key);
+    return false;
+}
+
+// ---- Gelarax
+bool ParseGelarax(const JsonValue &root, LayeredDesc &d)
+{
+    memset(&d.cfg, 0, sizeof(d.cfg));
+    if (!Need(root, "width", d.cfg.width, "config") || !Need(root, "vocab", d.cfg.vocab, "config")) return false;
+    const JsonValue *norm = root.Get("norm");
+    if (!norm || !Need(*norm, "eps", d.cfg.eps, "norm")) { if (!norm) EngineSetError("config.json: norm is missing"); return false; }
+    d.cfg.pos_base = 10000.0f;
+    const JsonValue *layers = root.Get("layers");
+    if (!layers || layers->type != JsonValue::Array || layers->arr.empty()) { EngineSetError("config.json: layers is missing or empty"); return false; }
+    for (size_t li = 0; li < layers->arr.size(); li++) {
+        const JsonValue &L = layers->arr[li];
+        ifa_layer_spec s; memset(&s, 0, sizeof(s));
+        std::vector<float> decay;
+        std::string type;
+        const JsonValue *mx = L.Get("mixer");
+        if (!L.GetString("type", type) || !mx || mx->type != JsonValue::Object) { EngineSetError("config.json: layer %zu has no type / mixer", li); return false; }
+        const std::string where = "layers[" + std::to_string(li) + "].mixer";
+        if (type == "parallel") {
+            s.mixer = IFA_MIX_WINDOW_LINEAR;
+            const JsonValue *a = mx->Get("left"), *r = mx->Get("right");
+            if (!a || !r) { EngineSetError("config.json: %s needs left and right", where.c_str()); return false; }
+            int vdim = 0;
+            const JsonValue *mask = a->Get("mask");
+            if (!mask) { EngineSetError("config.json: %s.left.mask is missing", where.c_str()); return false; }
+            if (!Need(*a, "heads", s.a_heads, "left") || !Need(*a, "kv_heads", s.a_kv_heads, "left") || !Need(*a, "dim", s.a_dim, "left") || !Need(*a, "vdim", vdim, "left")
+                || !Need(*a, "scale", s.a_scale, "left") || !Need(*a, "softcap", s.a_softcap, "left") || !Need(*a, "bias_max", s.a_bias_max, "left")
+                || !Need(*mask, "size", s.a_window, "left.mask") || !Need(*mask, "keep_first", s.a_keep_first, "left.mask")
+                || !Need(*mx, "left_scale", s.a_out_scale, "mixer") || !Need(*mx, "right_scale", s.l_out_scale, "mixer")
+                || !Need(*r, "heads", s.l_heads, "right") || !Need(*r, "dim", s.l_dim, "right") || !Need(*r, "vdim", s.l_vdim, "right")) return false;
+            if (vdim != s.a_dim) { EngineSetError("config.json: %s.left: the values are the keys, so vdim (%d) must equal dim (%d)", where.c_str(), vdim, s.a_dim); return false; }
+            const JsonValue *dc = r->Get("decay");
+            if (!dc || dc->type != JsonValue::Array || (int)dc->arr.size() != s.l_heads) { EngineSetError("config.json: %s.right.decay needs one value per head", where.c_str()); return false; }
+            for (const JsonValue &v : dc->arr) decay.push_back((float)v.num);
+        } else if (type == "delta") {
+            s.mixer = IFA_MIX_GATED_DELTA;
+            if (!Need(*mx, "heads", s.d_heads, "mixer") || !Need(*mx, "kv_heads", s.d_kv_heads, "mixer") || !Need(*mx, "dim", s.d_dim, "mixer")
+                || !Need(*mx, "vdim", s.d_vdim, "mixer") || !Need(*mx, "conv", s.d_conv, "mixer")) return false;
+        } else { EngineSetError("config.json: layer %zu: unknown type \"%s\"", li, type.c_str()); return false; }
+        const JsonValue *mlp = L.Get("mlp");
+        if (mlp && mlp->type == JsonValue::Object) {
+            std::string kind;
+            if (!mlp->GetString("kind", kind) || kind != "dense") { EngineSetError("config.json: layer %zu: mlp.kind \"%s\" is not supported (dense)", li, kind.c_str()); return false; }
+            if (!Need(*mlp, "ff", s.ffn, "mlp")) return false;
+        }
+        d.layers.push_back(s);
+        d.decays.push_back(decay);
+    }
+    d.cfg.n_layers = (int)d.layers.size();
+    return true;
+}
+
+struct NameId { const char *suffix; int id; };
+const NameId kGelaraxCommon[] = {{"norm1", IFA_LT_NORM1}, {"ls1", IFA_LT_LS1}, {"ls2", IFA_LT_LS2}, {"mlp.gate", IFA_LT_FFN_GATE}, {"mlp.gate.b", IFA_LT_FFN_GATE_B},
+                                 {"mlp.up", IFA_LT_FFN_UP}, {"mlp.up.b", IFA_LT_FFN_UP_B}, {"mlp.down", IFA_LT_FFN_DOWN}, {"mlp.down.b", IFA_LT_FFN_DOWN_B}};
+const NameId kGelaraxParallel[] = {{"mix.left.q", IFA_LT_A_Q}, {"mix.left.k", IFA_LT_A_K}, {"mix.left.rel", IFA_LT_A_REL}, {"mix.left.sink", IFA_LT_A_SINK},
+                                   {"mix.left.o", IFA_LT_A_O}, {"mix.right.q", IFA_LT_L_Q}, {"mix.right.k", IFA_LT_L_K}, {"mix.right.v", IFA_LT_L_V},
+                                   {"mix.right.g", IFA_LT_L_G}, {"mix.right.o", IFA_LT_L_O}, {"mix.right.norm", IFA_LT_L_NORM}};
+const NameId kGelaraxDelta[] = {{"mix.q", IFA_LT_D_Q}, {"mix.k", IFA_LT_D_K}, {"mix.v", IFA_LT_D_V}, {"mix.q.conv", IFA_LT_D_QCONV}, {"mix.k.conv", IFA_LT_D_KCONV},
+                                {"mix.v.conv", IFA_LT_D_VCONV}, {"mix.b", IFA_LT_D_B}, {"mix.a", IFA_LT_D_A}, {"mix.A_log", IFA_LT_D_ALOG},
+                                {"mix.dt_bias", IFA_LT_D_DTBIAS}, {"mix.g", IFA_LT_D_G}, {"mix.norm", IFA_LT_D_NORM}, {"mix.o", IFA_LT_D_O}};
+
+// tensor name -> (layer, id) for Gelarax: "embed", "final.norm", "head", "l<i>.<suffix>"
+void GelaraxNames(const LayeredDesc &d, std::vector<std::pair<std::string, std::pair<int, int>>> &out)
+{
+    out.push_back({"embed", {-1, IFA_T_EMBD}});
+    out.push_back({"final.norm", {-1, IFA_T_OUT_NORM}});
+    out.push_back({"head", {-1, IFA_T_LM_HEAD}});
+    for (size_t li = 0; li < d.layers.size(); li++) {
+        const std::string p = "l" + std::to_string(li) + ".";
+        for (const NameId &n : kGelaraxCommon) {
+            const bool ffn_part = n.id != IFA_LT_NORM1 && n.id != IFA_LT_LS1;
+            if (ffn_part && d.layers[li].ffn <= 0) continue;
+            out.push_back({p + n.suffix, {(int)li, n.id}});
+        }
+        if (d.layers[li].mixer == IFA_MIX_WINDOW_LINEAR) for (const NameId &n : kGelaraxParallel) out.push_back({p + n.suffix, {(int)li, n.id}});
+        else for (const NameId &n : kGelaraxDelta) out.push_back({p + n.suffix, {(int)li, n.id}});
+    }
+}
+
+// sizes that only a tensor's shape gives: the number of rows of a layer's distance-bias table
+bool GelaraxSizesFromTensors(const std::map<std::string, StTensorEntry> &index, LayeredDesc &d)
+{
+    for (size_t li = 0; li < d.layers.size(); li++) {
+        if (d.layers[li].mixer != IFA_MIX_WINDOW_LINEAR) continue;
+        const std::string name = "l" + std::to_string(li) + ".mix.left.rel";
+        auto it = index.find(name);
+        if (it == index.end() || it->second.shape.size() != 2 || it->second.shape[0] < 1) { EngineSetError("tensor %s is missing or not a matrix", name.c_str()); return false; }
+        d.layers[li].a_buckets = (int)it->second.shape[0];
+    }
+    return true;
+}
+
+struct ArchEntry {
+    const char *name;
+    bool (*parse)(const JsonValue &root, LayeredDesc &d);
+    bool (*sizes_from_tensors)(const std::map<std::string, StTensorEntry> &index, LayeredDesc &d);
+    void (*names)(const LayeredDesc &d, std::vector<std::pair<std::string, std::pair<int, int>>> &out);
+};
+const ArchEntry kArchitectures[] = {{"Gelarax", ParseGelarax, GelaraxSizesFromTensors, GelaraxNames}};
+
+const ArchEntry *FindArch(const std::string &name)
+{
+    for (const ArchEntry &a : kArchitectures) if (name == a.name) return &a;
+    return nullptr;
+}
+
+bool ParseDir(const ModelSpec &spec, LayeredDesc &d, const ArchEntry **arch)
+{
+    std::string text;
+    const std::string path = spec.dir + (spec.config_file.empty() ? "config.json" : spec.config_file);
+    if (!ReadText(path, text)) { EngineSetError("Cannot open %s", path.c_str()); return false; }
+    JsonValue root; JsonParser jp; std::string err;
+    if (!jp.Parse(text, root, &err) || root.type != JsonValue::Object) { EngineSetError("%s: %s", path.c_str(), err.c_str()); return false; }
+    std::string name;
+    root.GetString("architecture", name);
+    *arch = FindArch(name);
+    if (!*arch) { EngineSetError("%s: architecture \"%s\" is not registered", path.c_str(), name.c_str()); return false; }
+    return (*arch)->parse(root, d);
+}
+
+} // namespace
+
+bool LayeredArchitectureOf(const std::string &dir, std::string &arch)
+{
+    std::string text;
+    if (!ReadText(dir + "config.json", text)) return false;
+    JsonValue root; JsonParser jp;
+    if (!jp.Parse(text, root) || root.type != JsonValue::Object) return false;
+    return root.GetString("architecture", arch) && FindArch(arch) != nullptr;
+}
+
+// fills the spec of a layer-list model from its config.json (hyper-parameters for model_info; format "layered")
+bool LoadLayeredSpec(ModelSpec &spec)
+{
+    LayeredDesc d; const ArchEntry *arch = nullptr;
+    if (!ParseDir(spec, d, &arch)) return false;
+    spec.architecture = arch->name;
+    spec.network_structure = std::string("layered.") + arch->name;
+    spec.model_file_format = "layered";
+    if (spec.model_files.empty()) spec.model_files.push_back("model.safetensors");
+    spec.hyper_params.vocab_size = d.cfg.vocab; spec.hyper_params.embd_dims = d.cfg.width; spec.hyper_params.decoder_layers = d.cfg.n_layers;
+    spec.unk_token_id = -1;          // no vocabulary file: no id is withheld from selection
+    return true;
+}
+
+bool LoadLayered(std::vector<WorkerPlan> &plans, ModelSpec &spec)
+{
+    if (plans.size() != 1 || plans[0].n_stages > 1 || plans[0].tp_size > 1) { EngineSetError("model %s: layer-list models run on one device", spec.sid.c_str()); return false; }
+    LayeredDesc d; const ArchEntry *arch = nullptr;
+    if (!ParseDir(spec, d, &arch)) return false;
+    WorkerPlan &w = plans[0];
+    d.cfg.device = w.device;
+    d.cfg.max_ctx = spec.max_context_len > 0 ? spec.max_context_len : ModelSpec::DEFAULT_MAX_CONTEXT_LEN;
+    d.cfg.ops32 = spec.exact_fp32 ? 1 : 0;
+    w.layer0 = 0; w.layer1 = d.cfg.n_layers;
+    std::map<std::string, StTensorEntry> index;
+    for (const std::string &f : spec.model_files) if (!IndexSafetensorsFile(spec.dir + f, index)) return false;
+    if (!arch->sizes_from_tensors(index, d)) return false;
+    if (ifa_model_create_layered(&d.cfg, d.layers.data(), &w.model) != IFA_OK) { EngineSetError("ifa_model_create_layered: %s", ifa_last_error()); return false; }
+    std::vector<std::pair<std::string, std::pair<int, int>>> names;
+    arch->names(d, names);
+    std::vector<uint8_t> raw;
+    for (const auto &nm : names) {
+        auto it = index.find(nm.first);
+        if (it == index.end()) { EngineSetError("tensor %s is missing in %s", nm.first.c_str(), spec.dir.c_str()); return false; }
+        const StTensorEntry &e = it->second;
+        if (e.dtype != "BF16") { EngineSetError("tensor %s: dtype %s (bfloat16 expected)", nm.first.c_str(), e.dtype.c_str()); return false; }
+        size_t cnt = 1; for (size_t x : e.shape) cnt *= x;
+        if (e.end - e.begin != cnt * 2 || cnt == 0) { EngineSetError("tensor %s: %zu bytes for %zu values", nm.first.c_str(), e.end - e.begin, cnt); return false; }
+        raw.resize(cnt * 2);
+        FILE *fp = fopen(e.file.c_str(), "rb");
+        if (!fp) { EngineSetError("Failed to open file %s", e.file.c_str()); return false; }
+        fseek(fp, (long)(e.data_off + e.begin), SEEK_SET);
+        const bool ok = fread(raw.data(), 1, raw.size(), fp) == raw.size();
+        fclose(fp);
+        if (!ok) { EngineSetError("%s is truncated (tensor %s)", e.file.c_str(), nm.first.c_str()); return false; }
+        const size_t rows = e.shape.size() >= 2 ? e.shape[0] : 1, cols = e.shape.size() >= 2 ? cnt / e.shape[0] : cnt;
+        if (ifa_model_set_tensor_host(w.model, nm.second.first, nm.second.second, IFA_BF16, raw.data(), rows, cols) != IFA_OK) {
+            EngineSetError("tensor %s: %s", nm.first.c_str(), ifa_last_error()); return false;
+        }
+    }
+    for (size_t li = 0; li < d.layers.size(); li++)
+        if (d.layers[li].mixer == IFA_MIX_WINDOW_LINEAR
+            && ifa_model_set_tensor_host(w.model, (int)li, IFA_LT_L_DECAY, IFA_F32, d.decays[li].data(), 1, d.decays[li].size()) != IFA_OK) {
+            EngineSetError("layer %zu decay: %s", li, ifa_last_error()); return false;
+        }
+    return true;
+}
+
+} // namespace inferflow_amd

@@ -56,6 +56,7 @@ static uint16_t F32ToF16(float f)
     if (rem > 0x1000u || (rem == 0x1000u && (r & 1))) r++;
     return (uint16_t)(sign | r);
 }
+uint16_t FloatToHalfBits(float f) { return F32ToF16(f); }
 static float BF16ToF32(uint16_t b) { uint32_t x = (uint32_t)b << 16; float f; memcpy(&f, &x, 4); return f; }
 
 // ---------------------------------------------------------------- spec json
@@ -375,7 +376,7 @@ bool LoadLlama2DotC(std::vector<WorkerPlan> &plans, ModelSpec &spec)
 }
 
 // ------------------------------------------------------------- safetensors
-struct StEntry { std::string file; std::string dtype; std::vector<size_t> shape; size_t begin = 0, end = 0, data_off = 0; };
+typedef StTensorEntry StEntry;
 
 bool IndexSafetensors(const std::string &path, std::map<std::string, StEntry> &index)
 {
@@ -640,6 +641,8 @@ bool LoadSynthetic(std::vector<WorkerPlan> &plans, ModelSpec &spec)
 
 } // namespace
 
+bool IndexSafetensorsFile(const std::string &path, std::map<std::string, StTensorEntry> &index) { return IndexSafetensors(path, index); }
+
 bool BuildWorkers(std::vector<WorkerPlan> &plans, ModelSpec &spec)
 {
     for (WorkerPlan &w : plans) w.model = nullptr;
@@ -649,7 +652,8 @@ bool BuildWorkers(std::vector<WorkerPlan> &plans, ModelSpec &spec)
     if (fmt == "llama2.c" || fmt == "llama2_c") ok = LoadLlama2DotC(plans, spec);
     else if (fmt == "safetensors") ok = LoadSafetensors(plans, spec);
     else if (fmt == "synthetic") ok = LoadSynthetic(plans, spec);
-    else EngineSetError("model %s: model_file_format \"%s\" is not supported (llama2.c, safetensors, synthetic)", spec.sid.c_str(), fmt.c_str());
+    else if (fmt == "layered") ok = LoadLayered(plans, spec);
+    else EngineSetError("model %s: model_file_format \"%s\" is not supported (llama2.c, safetensors, synthetic, layered)", spec.sid.c_str(), fmt.c_str());
     for (WorkerPlan &w : plans)
         if (ok && ifa_model_finalize(w.model) != IFA_OK) { EngineSetError("ifa_model_finalize: %s", ifa_last_error()); ok = false; }
     if (!ok) for (WorkerPlan &w : plans) if (w.model) { ifa_model_destroy(w.model); w.model = nullptr; }
