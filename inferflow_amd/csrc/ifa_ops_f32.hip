@@ -10,14 +10,14 @@ namespace {
 // x[t][c] = embed[token_t][c] + pe(pos_t)[c];  pe[2i] = sin(p w_i), pe[2i + 1] = cos(p w_i), w_i = base^(-2i / width).
 // The angle of position p reaches hundreds of radians where one fp32 ulp is already 1e-4: it is formed in double.
 __global__ void __launch_bounds__(256) k_embed_sinpos(const bf16_t *__restrict__ embed, int vocab, int width, const int *__restrict__ tokens,
-                                                      const int *__restrict__ positions, float base_log, float *__restrict__ x)
+                                                      const int *__restrict__ positions, double base_log, float *__restrict__ x)
 {
     const int t = blockIdx.x;
     const int tok = min(max(tokens[t], 0), vocab - 1);
     const double p = (double)positions[t];
     for (int c = threadIdx.x; c < width; c += blockDim.x) {
         const int i2 = c & ~1;
-        const double w = exp(-(double)i2 / (double)width * (double)base_log);
+        const double w = exp(-(double)i2 / (double)width * base_log);
         const double a = p * w;
         const float pe = (float)((c & 1) ? cos(a) : sin(a));
         x[(size_t)t * width + c] = bf2f(embed[(size_t)tok * width + c]) + pe;
@@ -98,7 +98,7 @@ int ifa_embed_sinpos_f32(const void *embed_bf16, int vocab, int width, const int
     IFA_REQUIRE(embed_bf16 && tokens_dev && positions_dev && x_f32, "ifa_embed_sinpos_f32: null pointer");
     IFA_REQUIRE(vocab > 0 && width > 0 && tokens > 0 && base > 1.0f, "ifa_embed_sinpos_f32: bad shape");
     hipLaunchKernelGGL(k_embed_sinpos, dim3((unsigned)tokens), dim3(256), 0, ifa_s(stream), (const bf16_t *)embed_bf16, vocab, width, tokens_dev,
-                       positions_dev, logf(base), (float *)x_f32);
+                       positions_dev, log((double)base), (float *)x_f32);
     IFA_LAUNCH_CHECK();
     return IFA_OK;
 }

@@ -34,6 +34,30 @@ class InferenceEngine:
             raise EngineError("LoadConfig/Init failed: " + cls._err())
         return cls(h)
 
+    @classmethod
+    def from_model_dir(cls, model_dir, compute_dtype="bfloat16", max_context_len=1024, max_concurrent_queries=8, return_output_tensors=True):
+        """An engine for a bare model directory (config.json naming a registered layer-list architecture + model.safetensors)."""
+        h = _capi.lib().ifa_engine_create_from_dir(str(model_dir).encode(), compute_dtype.encode(), int(max_context_len), int(max_concurrent_queries),
+                                                   int(bool(return_output_tensors)))
+        if not h:
+            raise EngineError("LoadConfigForModelDir/Init failed: " + cls._err())
+        return cls(h)
+
+    def worker(self, rank=0):
+        """the ifa_model handle of partition rank `rank` as a c_void_p (for the ifa_model_* calls)"""
+        h = _capi.lib().ifa_engine_worker(self._h, int(rank))
+        return C.c_void_p(h) if h else None
+
+    def last_logits_f32(self, query_id):
+        """fp32 logits [rows, vocab] of the query's most recent step (return_output_tensors_f32; layer-list models)"""
+        rows, cols = C.c_int(0), C.c_int(0)
+        if not _capi.lib().ifa_engine_last_logits_f32(self._h, query_id, None, 0, C.byref(rows), C.byref(cols)):
+            raise EngineError(self._err())
+        out = np.zeros((rows.value, cols.value), np.float32)
+        if out.size:
+            _capi.lib().ifa_engine_last_logits_f32(self._h, query_id, out.ctypes.data_as(C.c_void_p), out.size, C.byref(rows), C.byref(cols))
+        return out
+
     def close(self):
         if self._h:
             _capi.lib().ifa_engine_destroy(self._h)
