@@ -370,6 +370,80 @@ def loopback_line(args):
     print(json.dumps(out), flush=True)
 
 
+ARCH_SIZES = {      # --arch gelarax: layer sizes that resemble a real model's, eight layers each (three windowed + linear attention, one delta rule, twice)
+    "w1024": dict(width=1024, ff=2816, heads=8, kv_heads=2, dim=128, lin_heads=8, delta_heads=8, delta_kv_heads=4),
+    "w2048": dict(width=2048, ff=5632, heads=16, kv_heads=4, dim=128, lin_heads=16, delta_heads=16, delta_kv_heads=8),
+}
+
+
+def run_arch_bench(args):
+    """--arch gelarax: prefill and decode throughput of Gelarax-shaped models with random bfloat16 weights (layer-list worker, fp32 residual) beside
+    the closest standard model of this framework at equal width / FFN / heads / layers (Llama wiring, F16 weights, F16 KV cache, same kernels as the
+    headline path with the quantiser switched off).  One JSON line; `value` = decode tokens/s of the largest Gelarax size."""
+    import shutil
+    import tempfile
+    import numpy as np
+    import torch
+    from inferflow_amd import dtypes as dt, synth
+    from inferflow_amd.engine import InferenceEngine
+    torch.cuda.set_device(0)
+    lens = [int(x) for x in args.prefill_lens.split(",") if x]
+    steps, warmup = args.steps, args.warmup
+    sizes = [x for x in args.arch_sizes.split(",") if x]
+    ctx = max(lens) + warmup + steps + 8
+    rng = np.random.default_rng(42)
+    rows = []
+
+    def timed(fn):
+        torch.cuda.synchronize(); t0 = time.perf_counter(); fn(); torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    for name in sizes:
+        sz = ARCH_SIZES[name]
+        cfg = synth.gelarax_config(vocab=32000, **sz)
+        d = tempfile.mkdtemp(prefix="ifa_gelarax_", dir="/dev/shm" if os.path.isdir("/dev/shm") else None)
+        try:
+            synth.write_gelarax_dir(d, cfg, seed=1)
+            eng = InferenceEngine.from_model_dir(d, "bfloat16", ctx, 2, False)
+        finally:
+            shutil.rmtree(d, ignore_errors=True)
+        g = {"prefill_tok_s": {}, "params": int(sum(int(np.prod(s)) for s in synth.gelarax_tensor_shapes(cfg).values()))}
+        for n in lens:
+            prompt = [int(t) for t in rng.integers(3, 32000, n)]
+            best = 1e9
+            for rep in range(3):
+                q = eng.add_query(prompt)
+                best = min(best, timed(lambda: eng.generate(q, 1)))
+                if rep < 2:
+                    eng.remove_query(q)
+            g["prefill_tok_s"][str(n)] = n / best
+        if warmup > 0:
+            eng.generate(q, warmup)
+        wall = timed(lambda: eng.generate(q, steps))
+        g["decode_tok_s"] = steps / wall; g["decode_ms_per_step"] = wall * 1e3 / steps; g["decode_context"] = "%d..%d" % (lens[-1] + warmup, lens[-1] + warmup + steps)
+        eng.close()
+        # the closest standard model: same width, FFN, heads and layer count, F16 weights
+        synth.SHAPES["cmp_" + name] = dict(dim=sz["width"], layers=8, heads=sz["heads"], kv_heads=sz["kv_heads"], head_dim=sz["dim"], ffn=sz["ff"], vocab=32000)
+        wk, _, _ = synth.build("cmp_" + name, dt.F16, dt.F16, ctx, quant_threshold=1 << 62)
+        c = {"prefill_tok_s": {}}
+        for n in lens:
+            prompt = rng.integers(3, 32000, n).astype(np.int32)
+            best = min(timed(lambda: wk.forward(prompt, 0)) for _ in range(3))
+            c["prefill_tok_s"][str(n)] = n / best
+        nxt = int(wk.forward(prompt, 0))
+        if warmup > 0:
+            wk.decode(nxt, lens[-1], warmup)
+        wall = timed(lambda: wk.decode(nxt, lens[-1] + warmup, steps))
+        c["decode_tok_s"] = steps / wall; c["decode_ms_per_step"] = wall * 1e3 / steps
+        del wk
+        rows.append({"size": name, "layers": 8, **sz, "gelarax": g, "closest_standard_model": c})
+    last = rows[-1]["gelarax"]
+    print(json.dumps({"metric": "decode tokens/sec, Gelarax-shaped model (%s), batch=1 greedy" % sizes[-1], "value": last["decode_tok_s"], "unit": "tokens/s", "n_gpus": 1,
+                      "steps": steps, "warmup": warmup, "ms_per_step": last["decode_ms_per_step"], "higher_is_better": True, "scaling": "strong", "vs_baseline": None,
+                      "dtype": "bf16 weights and matrix-product operands, f32 accumulation, residual and states", "data": "synthetic",
+                      "config": {"model": "Gelarax-shaped, random weights", "global_batch": 1, "seq_len": lens[-1], "parallelism": "single"}, "sizes": rows}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -388,7 +462,16 @@ def main():
                     "a functional check of the N > 1 step logic on a one-GPU box, not a scaling number")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=0, help="CPU baseline sample size (0 = auto)")
+    ap.add_argument("--arch", default="", help="'gelarax': instead of the headline workload, prefill / decode rates of Gelarax-shaped models beside the "
+                    "closest standard model at equal size (one GPU; --prefill-lens, --steps, --warmup apply)")
+    ap.add_argument("--arch-sizes", default="w1024,w2048")
     args = ap.parse_args()
+    if args.arch:
+        if args.arch.lower() != "gelarax":
+            raise SystemExit("unknown --arch %s (gelarax)" % args.arch)
+        if args.gpus > 1 or int(os.environ.get("WORLD_SIZE", "1")) > 1:
+            raise SystemExit("--arch runs on one GPU")
+        return run_arch_bench(args)
 
     import numpy as np
     import torch

@@ -505,11 +505,14 @@ int ifa_kv_store_f32(const void *k_f32, size_t ldk, const void *v_f32, size_t ld
 /* softmax attention of the step's rows over their sequences' caches: query i sees key j iff j <= i and (i - j < window or
  * j < keep_first); q RMS-normed per head if norm_q; score = q.k * scale, soft cap cap * tanh(score / cap) if softcap > 0, + bias
  * rel[bucket_of[i - j]][head] if rel (bf16 [n_buckets][heads], bucket_of_dev: int per distance 0 .. max_ctx - 1); sink_bf16 [heads]
- * (nullable): exp(sink) joins the denominator.  dim <= 256.  out fp32 [rows][heads * dim]. */
+ * (nullable): exp(sink) joins the denominator.  dim <= 256.  out fp32 [rows][heads * dim].
+ * Steps of at least tile_min_rows rows (head sizes 32 / 64 / 96 / 128) take the tiled kernel -- 128 queries of one sequence per workgroup,
+ * scores and weighted sums on the fp32 matrix cores -- which needs the step's sequences on the host too (seqs_host [n_seqs], the same
+ * values as seqs_dev; NULL / n_seqs 0: always one workgroup per row). */
 int ifa_attention_window_f32(const void *q_f32, size_t ldq, int heads, int kv_heads, int dim, int norm_q, float eps, float scale, float softcap,
                              int window, int keep_first, const void *rel_bf16, const int *bucket_of_dev, int n_buckets, const void *sink_bf16,
                              const void *seqs_dev, const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t k_off, size_t v_off,
-                             void *out_f32, size_t ldo, ifa_stream stream);
+                             void *out_f32, size_t ldo, const void *seqs_host, int n_seqs, int tile_min_rows, ifa_stream stream);
 
 /* ======================================================================== */
 /* Layer-list worker: a decoder whose layers are given one by one, each with its own sequence mixer, a 32-bit residual       */

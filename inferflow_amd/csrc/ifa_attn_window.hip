@@ -127,6 +127,145 @@ __global__ void __launch_bounds__(256) k_attn_window(WinAttnArgs P)
     }
 }
 
+
+// ---- prompts: 128 queries of one sequence per workgroup, the visible keys walked in blocks of 32 that are staged ONCE per workgroup
+// in LDS; each wave owns 32 queries: S = Q K^T and O += P V on the fp32 matrix cores (v_mfma_f32_32x32x2_f32: scores and weights
+// stay 32-bit), online softmax per query row (running maximum across the block's keys by lane exchange, the row sums kept per lane
+// and added up once at the end), P turned from the accumulator layout into an A operand through LDS.  dim = 32 NT.
+typedef float f32x16w __attribute__((ext_vector_type(16)));
+constexpr int WT_Q = 128, WT_K = 32;
+
+__device__ __forceinline__ float half_wave_max(float v)      // over the 32 lanes that share lane >> 5
+{
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+template <int NT>
+__global__ void __launch_bounds__(256) k_attn_window_tile(WinAttnArgs P, int n_seqs)
+{
+    constexpr int D = 32 * NT, DP = D + 1;
+    extern __shared__ float sm[];
+    float *Qs = sm;                          // [128][DP]
+    float *Ks = Qs + WT_Q * DP;              // [32][DP]
+    float *Vs = Ks + WT_K * DP;              // [32][DP]
+    float *Ps = Vs + WT_K * DP;              // [4][32][33]
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, i = lane & 31, g = lane >> 5;
+    const int h = blockIdx.y, kvh = h / (P.heads / P.kv_heads);
+    // which sequence and which of its 128-row tiles
+    int tile = blockIdx.x, sq = 0;
+    for (; sq < n_seqs; sq++) {
+        const int nt = (P.seqs[sq].n + WT_Q - 1) / WT_Q;
+        if (tile < nt) break;
+        tile -= nt;
+    }
+    if (sq >= n_seqs) return;
+    const SeqDesc sd = P.seqs[sq];
+    const int r0 = sd.row0 + tile * WT_Q, nq = min(WT_Q, sd.n - tile * WT_Q), p0 = sd.pos0 + tile * WT_Q;
+    const size_t kvd = (size_t)P.kv_heads * D;
+    const float *kc = P.slot_base[sd.slot] + P.k_off + (size_t)kvh * D, *vc = P.slot_base[sd.slot] + P.v_off + (size_t)kvh * D;
+    // Q rows of this wave, normed, into LDS
+    for (int rr = 0; rr < 32; rr++) {
+        const int q = 32 * wave + rr;
+        float v[NT > 2 ? 2 : 1];
+        float ssum = 0.0f;
+#pragma unroll
+        for (int e = 0; e < (NT > 2 ? 2 : 1); e++) {
+            const int c = lane + 64 * e;
+            v[e] = (q < nq && c < D) ? P.q[(size_t)(r0 + q) * P.ldq + (size_t)h * D + c] : 0.0f;
+            ssum = fmaf(v[e], v[e], ssum);
+        }
+        const float rinv = P.norm_q ? 1.0f / sqrtf(wave_sum(ssum) / (float)D + P.eps) : 1.0f;
+#pragma unroll
+        for (int e = 0; e < (NT > 2 ? 2 : 1); e++) { const int c = lane + 64 * e; if (c < D) Qs[q * DP + c] = v[e] * rinv; }
+    }
+    const int nq_w = min(32, max(0, nq - 32 * wave));             // queries of this wave
+    const int qlo = p0 + 32 * wave, qhi = qlo + nq_w - 1;          // their positions
+    const int lo_min = max(0, p0 - P.window + 1), nkeep = min(P.keep_first, lo_min), p_last = p0 + nq - 1;
+    const int nb_keep = (nkeep + WT_K - 1) / WT_K, nb_win = (p_last - lo_min + 1 + WT_K - 1) / WT_K;
+    f32x16w o[NT];
+    float m[16], l[16];
+#pragma unroll
+    for (int nt = 0; nt < NT; nt++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) o[nt][r] = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; r++) { m[r] = -INFINITY; l[r] = 0.0f; }
+    float *Pw = Ps + wave * 32 * 33;
+    for (int b = 0; b < nb_keep + nb_win; b++) {
+        const bool kept = b < nb_keep;
+        const int kb0 = kept ? b * WT_K : lo_min + (b - nb_keep) * WT_K;
+        const int kc_n = kept ? min(WT_K, nkeep - kb0) : min(WT_K, p_last - kb0 + 1);
+        __syncthreads();                 // the previous block's K / V reads are done (and Q is staged)
+        for (int e = tid; e < WT_K * (D / 4); e += 256) {
+            const int row = e / (D / 4), c4 = (e % (D / 4)) * 4;
+            float4 kv = make_float4(0.f, 0.f, 0.f, 0.f), vv = kv;
+            if (row < kc_n) {
+                kv = *reinterpret_cast<const float4 *>(kc + (size_t)(kb0 + row) * kvd + c4);
+                vv = *reinterpret_cast<const float4 *>(vc + (size_t)(kb0 + row) * kvd + c4);
+            }
+            float *kd = Ks + row * DP + c4, *vd = Vs + row * DP + c4;
+            kd[0] = kv.x; kd[1] = kv.y; kd[2] = kv.z; kd[3] = kv.w;
+            vd[0] = vv.x; vd[1] = vv.y; vd[2] = vv.z; vd[3] = vv.w;
+        }
+        __syncthreads();
+        const bool active = nq_w > 0 && kb0 <= qhi && (kept || kb0 + kc_n - 1 >= qlo - P.window + 1 || kb0 < P.keep_first);
+        if (active) {
+            f32x16w acc;
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[r] = 0.0f;
+            const float *qa = Qs + (32 * wave + i) * DP + g, *ka = Ks + i * DP + g;
+#pragma unroll 8
+            for (int s2 = 0; s2 < D / 2; s2++) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(qa[2 * s2], ka[2 * s2], acc, 0, 0, 0);
+            const int j = kb0 + i;
+            const bool jin = i < kc_n;
+#pragma unroll
+            for (int r = 0; r < 16; r++) {
+                const int q = (r & 3) + 8 * (r >> 2) + 4 * g, iq = qlo + q;
+                const bool vis = jin && q < nq_w && j <= iq && (iq - j < P.window || j < P.keep_first);
+                float sc = acc[r] * P.scale;
+                if (P.softcap > 0.0f) sc = P.softcap * tanhf(sc / P.softcap);
+                if (P.rel && vis) sc += bf2f(P.rel[(size_t)P.bucket_of[iq - j] * P.heads + h]);
+                sc = vis ? sc : -INFINITY;
+                const float m_new = fmaxf(m[r], half_wave_max(sc));
+                const float pr = vis ? expf(sc - m_new) : 0.0f;
+                const float corr = m[r] == -INFINITY ? 1.0f : expf(m[r] - m_new);      // (m_new == -inf only while nothing was visible: sums are 0)
+                l[r] = l[r] * corr + pr;
+                m[r] = m_new;
+#pragma unroll
+                for (int nt = 0; nt < NT; nt++) o[nt][r] *= corr;
+                Pw[q * 33 + i] = pr;
+            }
+        }
+        __syncthreads();                 // P of every wave is in LDS
+        if (active) {
+            const float *pa = Pw + i * 33 + g;
+#pragma unroll
+            for (int nt = 0; nt < NT; nt++) {
+                const float *va = Vs + g * DP + 32 * nt + i;
+#pragma unroll 8
+                for (int s2 = 0; s2 < WT_K / 2; s2++) o[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(pa[2 * s2], va[2 * s2 * DP], o[nt], 0, 0, 0);
+            }
+        }
+    }
+    const float snk = P.sink ? bf2f(P.sink[h]) : -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; r++) {
+        const int q = (r & 3) + 8 * (r >> 2) + 4 * g;
+        float ls = l[r];
+#pragma unroll
+        for (int of = 16; of > 0; of >>= 1) ls += __shfl_xor(ls, of, 64);
+        if (q >= nq_w) continue;
+        const float M = fmaxf(m[r], snk);
+        const float f = expf(m[r] - M);
+        const float L = ls * f + (P.sink ? expf(snk - M) : 0.0f);
+        const float sc = f / L;
+#pragma unroll
+        for (int nt = 0; nt < NT; nt++) P.out[(size_t)(r0 + 32 * wave + q) * P.ldo + (size_t)h * D + 32 * nt + i] = o[nt][r] * sc;
+    }
+}
+
 } // namespace
 
 extern "C" {
@@ -145,7 +284,7 @@ int ifa_kv_store_f32(const void *k_f32, size_t ldk, const void *v_f32, size_t ld
 int ifa_attention_window_f32(const void *q_f32, size_t ldq, int heads, int kv_heads, int dim, int norm_q, float eps, float scale, float softcap,
                              int window, int keep_first, const void *rel_bf16, const int *bucket_of_dev, int n_buckets, const void *sink_bf16,
                              const void *seqs_dev, const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t k_off, size_t v_off,
-                             void *out_f32, size_t ldo, ifa_stream stream)
+                             void *out_f32, size_t ldo, const void *seqs_host, int n_seqs, int tile_min_rows, ifa_stream stream)
 {
     IFA_REQUIRE(q_f32 && seqs_dev && row_seq_dev && slot_base_dev && out_f32, "ifa_attention_window_f32: null pointer");
     IFA_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && rows > 0 && window >= 1 && keep_first >= 0, "ifa_attention_window_f32: bad shape");
@@ -156,6 +295,21 @@ int ifa_attention_window_f32(const void *q_f32, size_t ldq, int heads, int kv_he
     P.softcap = softcap; P.window = window; P.keep_first = keep_first; P.rel = (const bf16_t *)rel_bf16; P.bucket_of = bucket_of_dev; P.n_buckets = n_buckets;
     P.sink = (const bf16_t *)sink_bf16; P.seqs = (const SeqDesc *)seqs_dev; P.row_seq = row_seq_dev; P.slot_base = (float *const *)slot_base_dev;
     P.k_off = k_off; P.v_off = v_off; P.out = (float *)out_f32; P.ldo = ldo;
+    // prompts: the tiled matrix-core kernel (head sizes 32 / 64 / 96 / 128, 16-byte aligned cache rows); single tokens and other sizes: a workgroup per row
+    if (rows >= (size_t)tile_min_rows && n_seqs > 0 && dim % 32 == 0 && dim <= 128 && k_off % 4 == 0 && v_off % 4 == 0) {
+        const ifa_seq_desc *sh = (const ifa_seq_desc *)seqs_host;
+        size_t tiles = 0;
+        for (int q = 0; q < n_seqs; q++) tiles += ((size_t)sh[q].n + WT_Q - 1) / WT_Q;
+        const int NT = dim / 32, DP = dim + 1;
+        const size_t smem_t = ((size_t)(WT_Q + 2 * WT_K) * DP + 4 * 32 * 33) * 4;
+        const dim3 grid((unsigned)tiles, (unsigned)heads);
+#define IFA_WT(N) { IFA_HIP_CHECK(hipFuncSetAttribute((const void *)k_attn_window_tile<N>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem_t)); \
+                    hipLaunchKernelGGL(k_attn_window_tile<N>, grid, dim3(256), smem_t, ifa_s(stream), P, n_seqs); }
+        if (NT == 1) IFA_WT(1) else if (NT == 2) IFA_WT(2) else if (NT == 3) IFA_WT(3) else IFA_WT(4)
+#undef IFA_WT
+        IFA_LAUNCH_CHECK();
+        return IFA_OK;
+    }
     const size_t smem = ((size_t)dim * 5 + 8) * 4;
     hipLaunchKernelGGL(k_attn_window, dim3((unsigned)rows, (unsigned)heads), dim3(256), smem, ifa_s(stream), P);
     IFA_LAUNCH_CHECK();

@@ -65,6 +65,8 @@ struct LayeredNet {
     size_t logits_rows = 0, logits_cap = 0;
     float *taps = nullptr; size_t taps_rows = 0; int opt_tap_layers = 0;
     int opt_graph = 1;
+    int opt_attn_tile_min = 16;            // steps of at least this many rows run the windowed attention through the tiled kernel
+    std::vector<ifa_seq_desc> seqs_host;   // the current step's sequences (the tiled attention's grid is sized from them)
     hipGraphExec_t step_exec = nullptr; hipGraph_t step_graph = nullptr; int step_slot = -1;
 };
 
@@ -217,7 +219,7 @@ int run_layers(ifa_model *m, size_t T, int nseq)
                                        L.o_k, L.o_v, s))) return rc;
             if ((rc = ifa_attention_window_f32(n->proj + L.c_aq, NI, sp.a_heads, sp.a_kv_heads, sp.a_dim, 1, c.eps, sp.a_scale, sp.a_softcap, sp.a_window,
                                                sp.a_keep_first, L.T(IFA_LT_A_REL).data, L.bucket_of, sp.a_buckets, L.T(IFA_LT_A_SINK).data, n->seqs_dev,
-                                               n->row_seq_dev, T, slots, L.o_k, L.o_v, n->m1, AQ, s))) return rc;
+                                               n->row_seq_dev, T, slots, L.o_k, L.o_v, n->m1, AQ, n->seqs_host.data(), (int)n->seqs_host.size(), n->opt_attn_tile_min, s))) return rc;
             if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_A_O).data, W, AQ, n->m1, AQ, T, nullptr, ls1, sp.a_out_scale, 1, n->x, W))) return rc;
             // decayed linear attention
             if ((rc = ifa_state_scan_f32(0, 1, n->proj + L.c_lq, NI, n->proj + L.c_lk, NI, n->proj + L.c_lv, NI, sp.l_heads, sp.l_heads, sp.l_dim, sp.l_vdim,
@@ -408,9 +410,10 @@ int lay_set_option(ifa_model *m, const char *name, int value)
 {
     LayeredNet *n = m->lay;
     if (!strcmp(name, "tap_layers")) { n->opt_tap_layers = value; drop_step_graph(n); return IFA_OK; }
+    if (!strcmp(name, "attn_tile_min")) { n->opt_attn_tile_min = value; return IFA_OK; }
     if (!strcmp(name, "graph")) { n->opt_graph = value; drop_step_graph(n); return IFA_OK; }
     if (!strcmp(name, "ops32")) { IFA_HIP_CHECK(hipStreamSynchronize(m->stream)); n->cfg.ops32 = value ? 1 : 0; drop_step_graph(n); return IFA_OK; }
-    return ifa_fail(IFA_ERR_ARG, "ifa_model_set_option: unknown option '%s' (layer-list model: tap_layers, graph, ops32)", name);
+    return ifa_fail(IFA_ERR_ARG, "ifa_model_set_option: unknown option '%s' (layer-list model: tap_layers, graph, ops32, attn_tile_min)", name);
 }
 
 int lay_set_excluded(ifa_model *m, const int *ids_host, int cnt)
@@ -452,6 +455,7 @@ int upload_tables(ifa_model *m, const std::vector<int> &tokens, const std::vecto
     memcpy(n->tab_pin + R, pos.data(), T * 4);
     memcpy(n->tab_pin + 2 * R, row_seq.data(), T * 4);
     memcpy(n->tab_pin + 3 * R, seqs.data(), S * sizeof(ifa_seq_desc));
+    n->seqs_host = seqs;
     IFA_HIP_CHECK(hipMemcpyAsync(n->tab_dev, n->tab_pin, (3 * R + 4 * S) * 4, hipMemcpyHostToDevice, m->stream));
     return IFA_OK;
 }

@@ -162,6 +162,91 @@ __global__ void __launch_bounds__(64) k_state_scan(ScanArgs P)
     if (live) for (int i = 0; i < dk; i++) state[(size_t)i * P.dv + j] = S[i * 64 + lane];
 }
 
+// The same recurrences with the column S[:, j] of a lane in REGISTERS (key sizes 32 / 64 / 128): q_t and k_t are broadcast from LDS
+// in 16-byte reads, so a token costs DK / 2 LDS reads and 2 DK (decay) or 3 DK (delta rule) fp32 operations per lane, against
+// 4 DK LDS accesses of the general kernel above.  Same order of operations per element: results are bit-identical to it.
+template <int KIND, int DK>
+__global__ void __launch_bounds__(64) k_state_scan_reg(ScanArgs P)
+{
+    __shared__ __attribute__((aligned(16))) float qs[DK], ks[DK];
+    const int seq = blockIdx.x / P.heads, h = blockIdx.x % P.heads;
+    const int lane = threadIdx.x, j = blockIdx.y * 64 + lane;
+    const bool live = j < P.dv;
+    const int jc = live ? j : P.dv - 1;
+    const int qh = h / (P.heads / P.qk_heads);
+    const SeqDesc sd = P.seqs[seq];
+    float *state = P.slot_base[sd.slot] + P.state_off + (size_t)h * DK * P.dv;
+    float S[DK];
+    if (sd.pos0 > 0) {
+#pragma unroll
+        for (int i = 0; i < DK; i++) S[i] = state[(size_t)i * P.dv + jc];
+    } else {
+#pragma unroll
+        for (int i = 0; i < DK; i++) S[i] = 0.0f;
+    }
+    const float dconst = KIND == 0 ? P.decay_head[h] : 0.0f;
+    constexpr int DKL = (DK + 63) / 64;
+    float qr[DKL], kr[DKL], vr, gr = 0.0f, br = 0.0f;
+    auto request = [&](int t) {
+        const size_t row = (size_t)(sd.row0 + t);
+#pragma unroll
+        for (int e = 0; e < DKL; e++) {
+            const int i = lane + 64 * e;
+            if (i < DK) {
+                qr[e] = P.q[row * P.ldq + (size_t)qh * DK + i]; kr[e] = P.k[row * P.ldk + (size_t)qh * DK + i];
+                if (P.in_act) { qr[e] = silu_exact(qr[e]); kr[e] = silu_exact(kr[e]); }
+            }
+        }
+        vr = P.v[row * P.ldv + (size_t)h * P.dv + jc];
+        if (P.in_act) vr = silu_exact(vr);
+        if (KIND == 1) { gr = P.decay_row[row * P.heads + h]; br = P.beta_row[row * P.heads + h]; }
+    };
+    if (sd.n > 0) request(0);
+    for (int t = 0; t < sd.n; t++) {
+        __syncthreads();
+#pragma unroll
+        for (int e = 0; e < DKL; e++) { const int i = lane + 64 * e; if (i < DK) { qs[i] = qr[e]; ks[i] = kr[e]; } }
+        const float vt = vr, gt = gr, bt = br;
+        __syncthreads();
+        if (t + 1 < sd.n) request(t + 1);
+        float o = 0.0f;
+        if (KIND == 0) {
+#pragma unroll
+            for (int i4 = 0; i4 < DK; i4 += 4) {
+                const float4 k4 = *reinterpret_cast<const float4 *>(ks + i4), q4 = *reinterpret_cast<const float4 *>(qs + i4);
+                S[i4] = fmaf(dconst, S[i4], k4.x * vt); o = fmaf(S[i4], q4.x, o);
+                S[i4 + 1] = fmaf(dconst, S[i4 + 1], k4.y * vt); o = fmaf(S[i4 + 1], q4.y, o);
+                S[i4 + 2] = fmaf(dconst, S[i4 + 2], k4.z * vt); o = fmaf(S[i4 + 2], q4.z, o);
+                S[i4 + 3] = fmaf(dconst, S[i4 + 3], k4.w * vt); o = fmaf(S[i4 + 3], q4.w, o);
+            }
+        } else {
+            float r = 0.0f;
+#pragma unroll
+            for (int i4 = 0; i4 < DK; i4 += 4) {
+                const float4 k4 = *reinterpret_cast<const float4 *>(ks + i4);
+                S[i4] *= gt; r = fmaf(S[i4], k4.x, r);
+                S[i4 + 1] *= gt; r = fmaf(S[i4 + 1], k4.y, r);
+                S[i4 + 2] *= gt; r = fmaf(S[i4 + 2], k4.z, r);
+                S[i4 + 3] *= gt; r = fmaf(S[i4 + 3], k4.w, r);
+            }
+            const float u = bt * (vt - r);
+#pragma unroll
+            for (int i4 = 0; i4 < DK; i4 += 4) {
+                const float4 k4 = *reinterpret_cast<const float4 *>(ks + i4), q4 = *reinterpret_cast<const float4 *>(qs + i4);
+                S[i4] = fmaf(k4.x, u, S[i4]); o = fmaf(S[i4], q4.x, o);
+                S[i4 + 1] = fmaf(k4.y, u, S[i4 + 1]); o = fmaf(S[i4 + 1], q4.y, o);
+                S[i4 + 2] = fmaf(k4.z, u, S[i4 + 2]); o = fmaf(S[i4 + 2], q4.z, o);
+                S[i4 + 3] = fmaf(k4.w, u, S[i4 + 3]); o = fmaf(S[i4 + 3], q4.w, o);
+            }
+        }
+        if (live) P.out[(size_t)(sd.row0 + t) * P.ldo + (size_t)h * P.dv + j] = o;
+    }
+    if (live) {
+#pragma unroll
+        for (int i = 0; i < DK; i++) state[(size_t)i * P.dv + j] = S[i];
+    }
+}
+
 // y[t][c] = o[t][c] / sqrt(mean_group(o^2) + eps) * w[c % wlen] * act(gate[t][c]); one workgroup per row, a wave per group
 __global__ void __launch_bounds__(256) k_gated_groupnorm(const float *__restrict__ o, size_t ldo, int C, int group, const bf16_t *__restrict__ w, int wlen,
                                                          const float *__restrict__ gate, size_t ldg, int gate_act, float eps, float *__restrict__ y,
@@ -244,6 +329,15 @@ int ifa_state_scan_f32(int kind, int in_act, const void *q_f32, size_t ldq, cons
     P.out = (float *)out_f32; P.ldo = ldo;
     const size_t smem = ((size_t)dk * 64 + 2 * (size_t)dk) * 4;
     const dim3 grid((unsigned)(n_seqs * heads), ifa_cdiv((size_t)dv, 64));
+#define IFA_SCAN_REG(DKV) \
+    if (dk == DKV) { \
+        if (kind == 0) hipLaunchKernelGGL((k_state_scan_reg<0, DKV>), grid, dim3(64), 0, ifa_s(stream), P); \
+        else hipLaunchKernelGGL((k_state_scan_reg<1, DKV>), grid, dim3(64), 0, ifa_s(stream), P); \
+        IFA_LAUNCH_CHECK(); \
+        return IFA_OK; \
+    }
+    IFA_SCAN_REG(32) IFA_SCAN_REG(64) IFA_SCAN_REG(128)
+#undef IFA_SCAN_REG
     if (kind == 0) {
         IFA_HIP_CHECK(hipFuncSetAttribute((const void *)k_state_scan<0>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
         hipLaunchKernelGGL(k_state_scan<0>, grid, dim3(64), smem, ifa_s(stream), P);

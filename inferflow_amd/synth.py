@@ -126,3 +126,77 @@ def weight_bytes(shape_name, wdtype=dt.Q4_B32T1A, quant_threshold=TENSOR_QUANT_T
 def kv_bytes_per_ctx_row(shape_name, kv_dtype=dt.F16):
     s = SHAPES[shape_name]
     return s["layers"] * 2 * dt.row_bytes(kv_dtype, s["kv_heads"] * s["head_dim"])
+
+
+# ---------------------------------------------------------------- layer-list models (Gelarax) with random weights
+def gelarax_config(width=2048, ff=5632, blocks=2, vocab=32000, heads=16, kv_heads=4, dim=128, window=1024, keep_first=4, lin_heads=16, lin_dim=64,
+                   lin_vdim=128, delta_heads=16, delta_kv_heads=8, delta_dim=128, delta_vdim=128, conv=4):
+    """`blocks` x (three windowed + linear attention layers, one gated delta rule layer), each with a gated feed-forward"""
+    par = {"type": "parallel",
+           "mixer": {"left": {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim, "scale": dim ** -0.5 * 8, "softcap": 30.0, "bias_max": 4 * window,
+                              "mask": {"size": window, "keep_first": keep_first}},
+                     "right": {"heads": lin_heads, "dim": lin_dim, "vdim": lin_vdim, "decay": [1.0 - 2.0 ** (-3 - 7 * i / max(1, lin_heads - 1)) for i in range(lin_heads)]},
+                     "left_scale": 1.0, "right_scale": 1.0},
+           "mlp": {"kind": "dense", "ff": ff}}
+    dl = {"type": "delta", "mixer": {"heads": delta_heads, "kv_heads": delta_kv_heads, "dim": delta_dim, "vdim": delta_vdim, "conv": conv},
+          "mlp": {"kind": "dense", "ff": ff}}
+    return {"architecture": "Gelarax", "width": width, "vocab": vocab, "norm": {"eps": 1e-6}, "layers": [par, par, par, dl] * blocks}
+
+
+def gelarax_tensor_shapes(cfg, buckets=32):
+    W_, V = cfg["width"], cfg["vocab"]
+    s = {"embed": (V, W_), "final.norm": (W_,), "head": (V, W_)}
+    for li, L in enumerate(cfg["layers"]):
+        p = "l%d." % li
+        s[p + "norm1"] = (W_,); s[p + "ls1"] = (W_,)
+        if L.get("mlp"):
+            F = L["mlp"]["ff"]
+            s.update({p + "ls2": (W_,), p + "mlp.gate": (F, W_), p + "mlp.gate.b": (F,), p + "mlp.up": (F, W_), p + "mlp.up.b": (F,), p + "mlp.down": (W_, F),
+                      p + "mlp.down.b": (W_,)})
+        m = L["mixer"]
+        if L["type"] == "parallel":
+            a, r = m["left"], m["right"]
+            s.update({p + "mix.left.q": (a["heads"] * a["dim"], W_), p + "mix.left.k": (a["kv_heads"] * a["dim"], W_), p + "mix.left.rel": (buckets, a["heads"]),
+                      p + "mix.left.sink": (a["heads"],), p + "mix.left.o": (W_, a["heads"] * a["dim"]),
+                      p + "mix.right.q": (r["heads"] * r["dim"], W_), p + "mix.right.k": (r["heads"] * r["dim"], W_), p + "mix.right.v": (r["heads"] * r["vdim"], W_),
+                      p + "mix.right.g": (r["heads"] * r["vdim"], W_), p + "mix.right.o": (W_, r["heads"] * r["vdim"]), p + "mix.right.norm": (r["heads"] * r["vdim"],)})
+        else:
+            qk, dv = m["kv_heads"] * m["dim"], m["heads"] * m["vdim"]
+            s.update({p + "mix.q": (qk, W_), p + "mix.k": (qk, W_), p + "mix.v": (dv, W_), p + "mix.q.conv": (qk, m["conv"]), p + "mix.k.conv": (qk, m["conv"]),
+                      p + "mix.v.conv": (dv, m["conv"]), p + "mix.b": (m["heads"], W_), p + "mix.a": (m["heads"], W_), p + "mix.A_log": (m["heads"],),
+                      p + "mix.dt_bias": (m["heads"],), p + "mix.g": (dv, W_), p + "mix.norm": (m["vdim"],), p + "mix.o": (W_, dv)})
+    return s
+
+
+def write_gelarax_dir(path, cfg, seed=0):
+    """config.json + model.safetensors (bfloat16, N(0, 1/fan_in) matrices, norm weights and layer scales near 1) for measurements"""
+    import json
+    import os
+    import struct
+    import numpy as np
+    os.makedirs(path, exist_ok=True)
+    with open(os.path.join(path, "config.json"), "w") as f:
+        json.dump(cfg, f)
+    rng = np.random.default_rng(seed)
+    shapes = gelarax_tensor_shapes(cfg)
+    header, off = {}, 0
+    for name, shape in shapes.items():
+        n = int(np.prod(shape)) * 2
+        header[name] = {"dtype": "BF16", "shape": list(shape), "data_offsets": [off, off + n]}
+        off += n
+    hj = json.dumps(header).encode()
+    hj += b" " * (-len(hj) % 8)
+    with open(os.path.join(path, "model.safetensors"), "wb") as f:
+        f.write(struct.pack("<Q", len(hj))); f.write(hj)
+        for name, shape in shapes.items():
+            leaf = name.split(".")[-1]
+            if len(shape) == 1 and leaf in ("norm1", "norm", "ls1", "ls2"):
+                a = 1.0 + 0.05 * rng.standard_normal(shape, dtype=np.float32)
+            elif leaf == "A_log":
+                a = rng.uniform(-3.0, 0.0, shape).astype(np.float32)
+            elif len(shape) == 1 or leaf in ("rel", "conv"):
+                a = 0.3 * rng.standard_normal(shape, dtype=np.float32)
+            else:
+                a = rng.standard_normal(shape, dtype=np.float32) * np.float32(1.0 / np.sqrt(shape[-1]))
+            f.write((np.ascontiguousarray(a).view(np.uint32) >> 16).astype(np.uint16).tobytes())
+    return path

@@ -203,8 +203,10 @@ def test_delta_gates_and_gated_group_norm():
         assert np.abs(y.cpu().numpy() - want.numpy()).max() < 1e-5
 
 
-@pytest.mark.parametrize("heads,kv_heads,dim,window,keep,nb,dmax", [(4, 2, 16, 9, 2, 8, 30), (2, 2, 8, 1, 0, 4, 6), (3, 1, 68, 300, 5, 32, 240), (6, 3, 32, 17, 40, 10, 12)])
-def test_windowed_attention_with_sink_cap_and_bucket_bias(heads, kv_heads, dim, window, keep, nb, dmax):
+@pytest.mark.parametrize("tile_min", [16, 1 << 30])       # prompts through the tiled matrix-core kernel / every row through the per-row kernel
+@pytest.mark.parametrize("heads,kv_heads,dim,window,keep,nb,dmax", [(4, 2, 16, 9, 2, 8, 30), (2, 2, 8, 1, 0, 4, 6), (3, 1, 68, 300, 5, 32, 240), (6, 3, 32, 17, 40, 10, 12),
+                                                                    (2, 1, 64, 20, 3, 8, 30), (2, 2, 128, 50, 0, 16, 100), (1, 1, 96, 9, 2, 8, 30), (4, 2, 64, 33, 33, 6, 7)])
+def test_windowed_attention_with_sink_cap_and_bucket_bias(heads, kv_heads, dim, window, keep, nb, dmax, tile_min):
     rng = np.random.default_rng(heads + dim + window)
     L, eps, scale, cap = 150, 1e-6, 0.3, 6.0
     q = rng.standard_normal((L, heads * dim + 4)).astype(np.float32)
@@ -227,7 +229,8 @@ def test_windowed_attention_with_sink_cap_and_bucket_bias(heads, kv_heads, dim, 
         ia.check(capi().ifa_kv_store_f32(p(kd), kv_heads * dim + 2, p(kd), kv_heads * dim + 2, kv_heads, dim, 1, eps, p(d), p(rs), T, p(sl.table), 0, ctx * kvd, stream()))
         out = torch.empty((T, heads * dim), dtype=torch.float32, device="cuda")
         ia.check(capi().ifa_attention_window_f32(p(dev32(q[at:at + n])), heads * dim + 4, heads, kv_heads, dim, 1, eps, scale, cap, window, keep, p(devbf(rel)),
-                                                 p(bucket_of), nb, p(devbf(sink)), p(d), p(rs), T, p(sl.table), 0, ctx * kvd, p(out), heads * dim, stream()))
+                                                 p(bucket_of), nb, p(devbf(sink)), p(d), p(rs), T, p(sl.table), 0, ctx * kvd, p(out), heads * dim,
+                                                 (C.c_int * 4)(0, n, at, 1), 1, tile_min, stream()))
         sync()
         assert np.abs(out.cpu().numpy() - want[at:at + n]).max() < 2e-5 * max(1.0, np.abs(want).max()), (at, n)
         at += n
@@ -236,5 +239,37 @@ def test_windowed_attention_with_sink_cap_and_bucket_bias(heads, kv_heads, dim, 
     d, rs, T = seq_tables([(1, L - 1, 1)])
     out = torch.empty((1, heads * dim), dtype=torch.float32, device="cuda")
     ia.check(capi().ifa_attention_window_f32(p(dev32(q[L - 1:])), heads * dim + 4, heads, kv_heads, dim, 1, eps, scale, cap, window, keep, p(devbf(rel)),
-                                             p(bucket_of), nb, None, p(d), p(rs), T, p(sl.table), 0, ctx * kvd, p(out), heads * dim, stream()))
+                                             p(bucket_of), nb, None, p(d), p(rs), T, p(sl.table), 0, ctx * kvd, p(out), heads * dim, None, 0, 0, stream()))
     assert np.abs(out.cpu().numpy() - want[L - 1:]).max() > 1e-4
+
+
+def test_windowed_attention_tiles_over_several_sequences():
+    """one step holds a 150-token prompt, a single continued token and a 40-token continued portion: tiles must not cross sequences"""
+    rng = np.random.default_rng(77)
+    heads, kv_heads, dim, window, keep, nb, dmax, eps, scale, cap = 4, 2, 32, 40, 2, 8, 60, 1e-6, 0.4, 8.0
+    L, ctx, kvd = 200, 208, kv_heads * dim
+    seq = {s_: (rng.standard_normal((L, heads * dim)).astype(np.float32), rng.standard_normal((L, kvd)).astype(np.float32)) for s_ in (0, 1, 2)}
+    rel, sink = orc.bf16_round(rng.standard_normal((nb, heads))), orc.bf16_round(rng.standard_normal(heads))
+    want = {s_: orc.windowed_attention(orc.t64(q), orc.t64(k), heads, kv_heads, dim, scale, cap, window, keep, orc.t64(rel), dmax, orc.t64(sink), eps).numpy()
+            for s_, (q, k) in seq.items()}
+    bucket_of = devi([orc.distance_bucket(n, nb, dmax) for n in range(ctx)])
+    sl = Slots(3, 2 * ctx * kvd)
+    at = {0: 0, 1: 0, 2: 0}
+    for step in ([(1, 30), (2, 100)], [(0, 150), (1, 1), (2, 40)], [(2, 60), (0, 50), (1, 129)]):
+        seqs = [(n, at[s_], s_) for s_, n in step]
+        d, rs, T = seq_tables(seqs)
+        kd = dev32(np.concatenate([seq[s_][1][at[s_]:at[s_] + n] for s_, n in step], 0))
+        qd = dev32(np.concatenate([seq[s_][0][at[s_]:at[s_] + n] for s_, n in step], 0))
+        ia.check(capi().ifa_kv_store_f32(p(kd), kvd, p(kd), kvd, kv_heads, dim, 1, eps, p(d), p(rs), T, p(sl.table), 0, ctx * kvd, stream()))
+        out = torch.empty((T, heads * dim), dtype=torch.float32, device="cuda")
+        host, r = [], 0
+        for n, pos0, slot in seqs:
+            host += [r, n, pos0, slot]; r += n
+        ia.check(capi().ifa_attention_window_f32(p(qd), heads * dim, heads, kv_heads, dim, 1, eps, scale, cap, window, keep, p(devbf(rel)), p(bucket_of), nb,
+                                                 p(devbf(sink)), p(d), p(rs), T, p(sl.table), 0, ctx * kvd, p(out), heads * dim, (C.c_int * len(host))(*host),
+                                                 len(seqs), 16, stream()))
+        sync()
+        got, r = out.cpu().numpy(), 0
+        for s_, n in step:
+            assert np.abs(got[r:r + n] - want[s_][at[s_]:at[s_] + n]).max() < 2e-5 * max(1.0, np.abs(want[s_]).max()), (s_, at[s_], n)
+            r += n; at[s_] += n
