@@ -508,11 +508,12 @@ int ifa_kv_store_f32(const void *k_f32, size_t ldk, const void *v_f32, size_t ld
  * (nullable): exp(sink) joins the denominator.  dim <= 256.  out fp32 [rows][heads * dim].
  * Steps of at least tile_min_rows rows (head sizes 32 / 64 / 96 / 128) take the tiled kernel -- 128 queries of one sequence per workgroup,
  * scores and weighted sums on the fp32 matrix cores -- which needs the step's sequences on the host too (seqs_host [n_seqs], the same
- * values as seqs_dev; NULL / n_seqs 0: always one workgroup per row). */
+ * values as seqs_dev; NULL / n_seqs 0: always one workgroup per row).  With a workspace (ws_f32, ws_bytes; nullable) and at most 512
+ * (row, head) pairs, the keys of a pair are shared out to up to 16 workgroups and merged by a second launch (decode steps). */
 int ifa_attention_window_f32(const void *q_f32, size_t ldq, int heads, int kv_heads, int dim, int norm_q, float eps, float scale, float softcap,
                              int window, int keep_first, const void *rel_bf16, const int *bucket_of_dev, int n_buckets, const void *sink_bf16,
                              const void *seqs_dev, const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t k_off, size_t v_off,
-                             void *out_f32, size_t ldo, const void *seqs_host, int n_seqs, int tile_min_rows, ifa_stream stream);
+                             void *out_f32, size_t ldo, const void *seqs_host, int n_seqs, int tile_min_rows, void *ws_f32, size_t ws_bytes, ifa_stream stream);
 
 /* ======================================================================== */
 /* Layer-list worker: a decoder whose layers are given one by one, each with its own sequence mixer, a 32-bit residual       */

@@ -160,7 +160,7 @@ SIGNATURES = {
     "ifa_state_scan_f32": (_i, [_i, _i, _vp, _sz, _vp, _sz, _vp, _sz, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _sz, _vp, _sz, _vp]),
     "ifa_gated_groupnorm_f32": (_i, [_vp, _sz, _sz, _i, _i, _vp, _i, _vp, _sz, _i, _f, _vp, _sz, _vp]),
     "ifa_kv_store_f32": (_i, [_vp, _sz, _vp, _sz, _i, _i, _i, _f, _vp, _vp, _sz, _vp, _sz, _sz, _vp]),
-    "ifa_attention_window_f32": (_i, [_vp, _sz, _i, _i, _i, _i, _f, _f, _f, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _sz, _vp, _sz, _sz, _vp, _sz, _vp, _i, _i, _vp]),
+    "ifa_attention_window_f32": (_i, [_vp, _sz, _i, _i, _i, _i, _f, _f, _f, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _sz, _vp, _sz, _sz, _vp, _sz, _vp, _i, _i, _vp, _sz, _vp]),
     "ifa_model_create_layered": (_i, [_vp, _vp, C.POINTER(_vp)]),
     "ifa_model_set_tensor_host": (_i, [_vp, _i, _i, _i, _vp, _sz, _sz]),
     "ifa_model_logits_f32": (_i, [_vp, C.POINTER(_vp), C.POINTER(_sz), C.POINTER(_sz)]),

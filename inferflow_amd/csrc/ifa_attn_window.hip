@@ -6,6 +6,7 @@
 //   * a sink per head: exp(sink) joins the denominator, with no key and no value
 // Scores, weights and sums are fp32.  The cache rows are [max_ctx][kv_heads * dim] per (slot, layer): K holds the normed keys,
 // V the values; a row is addressed by its true position, so kept first tokens keep their distances.
+#include <algorithm>
 #include "ifa_host.h"
 #include "ifa_f32_common.h"
 
@@ -43,6 +44,7 @@ struct WinAttnArgs {
     const bf16_t *sink;                                          // [heads] or null
     const SeqDesc *seqs; const int *row_seq; float *const *slot_base; size_t k_off, v_off;
     float *out; size_t ldo;
+    float *ws; int nsplit;           // nsplit > 1: the keys of a (row, head) are shared out to nsplit workgroups; partial results in ws [rows][heads][nsplit][dim + 2]
 };
 
 constexpr int WA_DPL = 4;         // dim <= 64 * WA_DPL
@@ -76,7 +78,8 @@ __global__ void __launch_bounds__(256) k_attn_window(WinAttnArgs P)
 #pragma unroll
     for (int e = 0; e < WA_DPL; e++) acc[e] = 0.0f;
     const int nchunks = (nk + 63) / 64;
-    for (int ch = wave; ch < nchunks; ch += 4) {
+    const int nsplit = max(1, P.nsplit), split = blockIdx.z;
+    for (int ch = split * 4 + wave; ch < nchunks; ch += 4 * nsplit) {
         const int vi = ch * 64 + lane;
         const bool valid = vi < nk;
         const int j = valid ? (vi < nkeep ? vi : lo + (vi - nkeep)) : i;
@@ -114,6 +117,20 @@ __global__ void __launch_bounds__(256) k_attn_window(WinAttnArgs P)
 #pragma unroll
     for (int e = 0; e < WA_DPL; e++) { const int d = lane + 64 * e; if (d < dim) wacc[wave * dim + d] = acc[e]; }
     __syncthreads();
+    if (nsplit > 1) {      // this workgroup's share: maximum, sum and weighted values relative to that maximum; the sink joins in the combine
+        float M = -INFINITY;
+        for (int w = 0; w < 4; w++) M = fmaxf(M, wm[w]);
+        float L = 0.0f, f[4];
+        for (int w = 0; w < 4; w++) { f[w] = wm[w] == -INFINITY ? 0.0f : expf(wm[w] - M); L += wl[w] * f[w]; }
+        float *dst = P.ws + (((size_t)t * P.heads + h) * nsplit + split) * (dim + 2);
+        if (tid == 0) { dst[0] = M; dst[1] = L; }
+        for (int d = tid; d < dim; d += blockDim.x) {
+            float o = 0.0f;
+            for (int w = 0; w < 4; w++) o = fmaf(wacc[w * dim + d], f[w], o);
+            dst[2 + d] = o;
+        }
+        return;
+    }
     const float snk = P.sink ? bf2f(P.sink[h]) : -INFINITY;
     float M = snk;
     for (int w = 0; w < 4; w++) M = fmaxf(M, wm[w]);
@@ -123,6 +140,23 @@ __global__ void __launch_bounds__(256) k_attn_window(WinAttnArgs P)
     for (int d = tid; d < dim; d += blockDim.x) {
         float o = 0.0f;
         for (int w = 0; w < 4; w++) o = fmaf(wacc[w * dim + d], f[w], o);
+        P.out[(size_t)t * P.ldo + (size_t)h * dim + d] = o / L;
+    }
+}
+
+// grid (rows, heads): the shares of a (row, head) and its sink into the output row
+__global__ void __launch_bounds__(64) k_attn_window_combine(WinAttnArgs P)
+{
+    const int t = blockIdx.x, h = blockIdx.y, dim = P.dim, nsplit = P.nsplit;
+    const float *src = P.ws + ((size_t)t * P.heads + h) * nsplit * (dim + 2);
+    const float snk = P.sink ? bf2f(P.sink[h]) : -INFINITY;
+    float M = snk;
+    for (int sp = 0; sp < nsplit; sp++) M = fmaxf(M, src[(size_t)sp * (dim + 2)]);
+    float L = P.sink ? expf(snk - M) : 0.0f;
+    for (int sp = 0; sp < nsplit; sp++) { const float m = src[(size_t)sp * (dim + 2)]; if (m != -INFINITY) L += src[(size_t)sp * (dim + 2) + 1] * expf(m - M); }
+    for (int d = threadIdx.x; d < dim; d += blockDim.x) {
+        float o = 0.0f;
+        for (int sp = 0; sp < nsplit; sp++) { const float m = src[(size_t)sp * (dim + 2)]; if (m != -INFINITY) o = fmaf(src[(size_t)sp * (dim + 2) + 2 + d], expf(m - M), o); }
         P.out[(size_t)t * P.ldo + (size_t)h * dim + d] = o / L;
     }
 }
@@ -284,7 +318,7 @@ int ifa_kv_store_f32(const void *k_f32, size_t ldk, const void *v_f32, size_t ld
 int ifa_attention_window_f32(const void *q_f32, size_t ldq, int heads, int kv_heads, int dim, int norm_q, float eps, float scale, float softcap,
                              int window, int keep_first, const void *rel_bf16, const int *bucket_of_dev, int n_buckets, const void *sink_bf16,
                              const void *seqs_dev, const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t k_off, size_t v_off,
-                             void *out_f32, size_t ldo, const void *seqs_host, int n_seqs, int tile_min_rows, ifa_stream stream)
+                             void *out_f32, size_t ldo, const void *seqs_host, int n_seqs, int tile_min_rows, void *ws_f32, size_t ws_bytes, ifa_stream stream)
 {
     IFA_REQUIRE(q_f32 && seqs_dev && row_seq_dev && slot_base_dev && out_f32, "ifa_attention_window_f32: null pointer");
     IFA_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && rows > 0 && window >= 1 && keep_first >= 0, "ifa_attention_window_f32: bad shape");
@@ -294,7 +328,7 @@ int ifa_attention_window_f32(const void *q_f32, size_t ldq, int heads, int kv_he
     P.q = (const float *)q_f32; P.ldq = ldq; P.heads = heads; P.kv_heads = kv_heads; P.dim = dim; P.norm_q = norm_q; P.eps = eps; P.scale = scale;
     P.softcap = softcap; P.window = window; P.keep_first = keep_first; P.rel = (const bf16_t *)rel_bf16; P.bucket_of = bucket_of_dev; P.n_buckets = n_buckets;
     P.sink = (const bf16_t *)sink_bf16; P.seqs = (const SeqDesc *)seqs_dev; P.row_seq = row_seq_dev; P.slot_base = (float *const *)slot_base_dev;
-    P.k_off = k_off; P.v_off = v_off; P.out = (float *)out_f32; P.ldo = ldo;
+    P.k_off = k_off; P.v_off = v_off; P.out = (float *)out_f32; P.ldo = ldo; P.ws = nullptr; P.nsplit = 1;
     // prompts: the tiled matrix-core kernel (head sizes 32 / 64 / 96 / 128, 16-byte aligned cache rows); single tokens and other sizes: a workgroup per row
     if (rows >= (size_t)tile_min_rows && n_seqs > 0 && dim % 32 == 0 && dim <= 128 && k_off % 4 == 0 && v_off % 4 == 0) {
         const ifa_seq_desc *sh = (const ifa_seq_desc *)seqs_host;
@@ -311,7 +345,15 @@ int ifa_attention_window_f32(const void *q_f32, size_t ldq, int heads, int kv_he
         return IFA_OK;
     }
     const size_t smem = ((size_t)dim * 5 + 8) * 4;
-    hipLaunchKernelGGL(k_attn_window, dim3((unsigned)rows, (unsigned)heads), dim3(256), smem, ifa_s(stream), P);
+    // few rows: a (row, head)'s keys are shared out to several workgroups (one workgroup pulls its keys through ONE compute unit)
+    int nsplit = 1;
+    if (ws_f32 && rows * (size_t)heads <= 512) {
+        nsplit = (int)std::min<size_t>(16, ((size_t)window + (size_t)keep_first + 255) / 256);
+        while (nsplit > 1 && rows * (size_t)heads * nsplit * ((size_t)dim + 2) * 4 > ws_bytes) nsplit--;
+    }
+    P.ws = (float *)ws_f32; P.nsplit = nsplit;
+    hipLaunchKernelGGL(k_attn_window, dim3((unsigned)rows, (unsigned)heads, (unsigned)nsplit), dim3(256), smem, ifa_s(stream), P);
+    if (nsplit > 1) hipLaunchKernelGGL(k_attn_window_combine, dim3((unsigned)rows, (unsigned)heads), dim3(64), 0, ifa_s(stream), P);
     IFA_LAUNCH_CHECK();
     return IFA_OK;
 }

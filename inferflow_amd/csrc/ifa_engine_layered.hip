@@ -65,6 +65,7 @@ struct LayeredNet {
     size_t logits_rows = 0, logits_cap = 0;
     float *taps = nullptr; size_t taps_rows = 0; int opt_tap_layers = 0;
     int opt_graph = 1;
+    float *attn_ws = nullptr; size_t attn_ws_bytes = 0;      // partial results of the windowed attention when a (row, head)'s keys are shared out
     int opt_attn_tile_min = 16;            // steps of at least this many rows run the windowed attention through the tiled kernel
     std::vector<ifa_seq_desc> seqs_host;   // the current step's sequences (the tiled attention's grid is sized from them)
     hipGraphExec_t step_exec = nullptr; hipGraph_t step_graph = nullptr; int step_slot = -1;
@@ -219,7 +220,7 @@ int run_layers(ifa_model *m, size_t T, int nseq)
                                        L.o_k, L.o_v, s))) return rc;
             if ((rc = ifa_attention_window_f32(n->proj + L.c_aq, NI, sp.a_heads, sp.a_kv_heads, sp.a_dim, 1, c.eps, sp.a_scale, sp.a_softcap, sp.a_window,
                                                sp.a_keep_first, L.T(IFA_LT_A_REL).data, L.bucket_of, sp.a_buckets, L.T(IFA_LT_A_SINK).data, n->seqs_dev,
-                                               n->row_seq_dev, T, slots, L.o_k, L.o_v, n->m1, AQ, n->seqs_host.data(), (int)n->seqs_host.size(), n->opt_attn_tile_min, s))) return rc;
+                                               n->row_seq_dev, T, slots, L.o_k, L.o_v, n->m1, AQ, n->seqs_host.data(), (int)n->seqs_host.size(), n->opt_attn_tile_min, n->attn_ws, n->attn_ws_bytes, s))) return rc;
             if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_A_O).data, W, AQ, n->m1, AQ, T, nullptr, ls1, sp.a_out_scale, 1, n->x, W))) return rc;
             // decayed linear attention
             if ((rc = ifa_state_scan_f32(0, 1, n->proj + L.c_lq, NI, n->proj + L.c_lk, NI, n->proj + L.c_lv, NI, sp.l_heads, sp.l_heads, sp.l_dim, sp.l_vdim,
@@ -282,6 +283,7 @@ int lay_destroy(ifa_model *m)
     for (float *p : n->slot_ptr) lay_free(p);
     lay_free(n->slot_base_dev);
     if (n->tab_pin) (void)hipHostFree(n->tab_pin);
+    lay_free(n->attn_ws);
     lay_free(n->tab_dev); lay_free(n->excl_dev); lay_free(n->next_dev); lay_free(n->ring_dev);
     float *bufs[] = {n->x, n->h, n->proj, n->m1, n->m2, n->m3, n->beta, n->decay, n->logits, n->taps};
     for (float *b : bufs) lay_free(b);
@@ -372,6 +374,13 @@ int lay_finalize(ifa_model *m)
             LTensor &t = L.T(id);
             if (t.data) { lay_free(t.data); t.data = nullptr; }
         }
+    }
+    if (!n->attn_ws) {
+        size_t per_row = 0;
+        for (const LLayer &L : n->layers)
+            if (L.spec.mixer == IFA_MIX_WINDOW_LINEAR) per_row = std::max(per_row, (size_t)L.spec.a_heads * 16 * ((size_t)L.spec.a_dim + 2) * 4);
+        n->attn_ws_bytes = per_row * 64;
+        if (n->attn_ws_bytes) IFA_HIP_CHECK(hipMalloc((void **)&n->attn_ws, n->attn_ws_bytes));
     }
     if (!n->slot_base_dev) {
         n->arena_floats = off;

@@ -162,13 +162,18 @@ __global__ void __launch_bounds__(64) k_state_scan(ScanArgs P)
     if (live) for (int i = 0; i < dk; i++) state[(size_t)i * P.dv + j] = S[i * 64 + lane];
 }
 
-// The same recurrences with the column S[:, j] of a lane in REGISTERS (key sizes 32 / 64 / 128): q_t and k_t are broadcast from LDS
-// in 16-byte reads, so a token costs DK / 2 LDS reads and 2 DK (decay) or 3 DK (delta rule) fp32 operations per lane, against
-// 4 DK LDS accesses of the general kernel above.  Same order of operations per element: results are bit-identical to it.
+// The same recurrences with the column S[:, j] of a lane in REGISTERS (key sizes 32 / 64 / 128).  Tokens go in groups of 8: the
+// group's q, k (and gates) sit in LDS and are broadcast in 16-byte reads, the NEXT group's operands are requested from memory before
+// the current group is computed (a token is ~0.3 us of dependent arithmetic; a memory round trip is longer than that).  A token costs
+// DK / 2 LDS reads and 2 DK (decay) or 3 DK (delta rule) fp32 operations per lane.  Same order of operations per element as the
+// general kernel above: bit-identical results.
+constexpr int SCAN_TB = 8;
+
 template <int KIND, int DK>
 __global__ void __launch_bounds__(64) k_state_scan_reg(ScanArgs P)
 {
-    __shared__ __attribute__((aligned(16))) float qs[DK], ks[DK];
+    __shared__ __attribute__((aligned(16))) float qs[2][SCAN_TB][DK], ks[2][SCAN_TB][DK];
+    __shared__ float gs[2][SCAN_TB], bs[2][SCAN_TB];
     const int seq = blockIdx.x / P.heads, h = blockIdx.x % P.heads;
     const int lane = threadIdx.x, j = blockIdx.y * 64 + lane;
     const bool live = j < P.dv;
@@ -185,61 +190,78 @@ __global__ void __launch_bounds__(64) k_state_scan_reg(ScanArgs P)
         for (int i = 0; i < DK; i++) S[i] = 0.0f;
     }
     const float dconst = KIND == 0 ? P.decay_head[h] : 0.0f;
-    constexpr int DKL = (DK + 63) / 64;
-    float qr[DKL], kr[DKL], vr, gr = 0.0f, br = 0.0f;
-    auto request = [&](int t) {
-        const size_t row = (size_t)(sd.row0 + t);
+    constexpr int PER = SCAN_TB * DK / 64;          // q (and k) values of a group per lane
+    float qr[PER], kr[PER], vnext[SCAN_TB], vcur[SCAN_TB], gr = 0.0f, br = 0.0f;
+    auto request = [&](int t0) {                    // the group that starts at token t0 -> registers
 #pragma unroll
-        for (int e = 0; e < DKL; e++) {
-            const int i = lane + 64 * e;
-            if (i < DK) {
-                qr[e] = P.q[row * P.ldq + (size_t)qh * DK + i]; kr[e] = P.k[row * P.ldk + (size_t)qh * DK + i];
-                if (P.in_act) { qr[e] = silu_exact(qr[e]); kr[e] = silu_exact(kr[e]); }
-            }
+        for (int u = 0; u < PER; u++) {
+            const int e = lane + 64 * u, tt = e / DK, i = e % DK;
+            const size_t row = (size_t)(sd.row0 + min(t0 + tt, sd.n - 1));
+            qr[u] = P.q[row * P.ldq + (size_t)qh * DK + i]; kr[u] = P.k[row * P.ldk + (size_t)qh * DK + i];
+            if (P.in_act) { qr[u] = silu_exact(qr[u]); kr[u] = silu_exact(kr[u]); }
         }
-        vr = P.v[row * P.ldv + (size_t)h * P.dv + jc];
-        if (P.in_act) vr = silu_exact(vr);
-        if (KIND == 1) { gr = P.decay_row[row * P.heads + h]; br = P.beta_row[row * P.heads + h]; }
+#pragma unroll
+        for (int tt = 0; tt < SCAN_TB; tt++) {
+            const size_t row = (size_t)(sd.row0 + min(t0 + tt, sd.n - 1));
+            vnext[tt] = P.v[row * P.ldv + (size_t)h * P.dv + jc];
+            if (P.in_act) vnext[tt] = silu_exact(vnext[tt]);
+        }
+        if (KIND == 1 && lane < SCAN_TB) {
+            const size_t row = (size_t)(sd.row0 + min(t0 + lane, sd.n - 1));
+            gr = P.decay_row[row * P.heads + h]; br = P.beta_row[row * P.heads + h];
+        }
     };
-    if (sd.n > 0) request(0);
-    for (int t = 0; t < sd.n; t++) {
-        __syncthreads();
+    auto publish = [&](int buf) {                   // registers -> LDS buffer
 #pragma unroll
-        for (int e = 0; e < DKL; e++) { const int i = lane + 64 * e; if (i < DK) { qs[i] = qr[e]; ks[i] = kr[e]; } }
-        const float vt = vr, gt = gr, bt = br;
-        __syncthreads();
-        if (t + 1 < sd.n) request(t + 1);
-        float o = 0.0f;
-        if (KIND == 0) {
+        for (int u = 0; u < PER; u++) { const int e = lane + 64 * u; qs[buf][e / DK][e % DK] = qr[u]; ks[buf][e / DK][e % DK] = kr[u]; }
+        if (KIND == 1 && lane < SCAN_TB) { gs[buf][lane] = gr; bs[buf][lane] = br; }
 #pragma unroll
-            for (int i4 = 0; i4 < DK; i4 += 4) {
-                const float4 k4 = *reinterpret_cast<const float4 *>(ks + i4), q4 = *reinterpret_cast<const float4 *>(qs + i4);
-                S[i4] = fmaf(dconst, S[i4], k4.x * vt); o = fmaf(S[i4], q4.x, o);
-                S[i4 + 1] = fmaf(dconst, S[i4 + 1], k4.y * vt); o = fmaf(S[i4 + 1], q4.y, o);
-                S[i4 + 2] = fmaf(dconst, S[i4 + 2], k4.z * vt); o = fmaf(S[i4 + 2], q4.z, o);
-                S[i4 + 3] = fmaf(dconst, S[i4 + 3], k4.w * vt); o = fmaf(S[i4 + 3], q4.w, o);
+        for (int tt = 0; tt < SCAN_TB; tt++) vcur[tt] = vnext[tt];
+    };
+    if (sd.n > 0) { request(0); publish(0); }
+    __syncthreads();
+    for (int t0 = 0, buf = 0; t0 < sd.n; t0 += SCAN_TB, buf ^= 1) {
+        const bool more = t0 + SCAN_TB < sd.n;
+        if (more) request(t0 + SCAN_TB);
+        const int cnt = min(SCAN_TB, sd.n - t0);
+        for (int tt = 0; tt < cnt; tt++) {
+            const float vt = vcur[tt];
+            const float *kq = ks[buf][tt], *qq = qs[buf][tt];
+            float o = 0.0f;
+            if (KIND == 0) {
+#pragma unroll
+                for (int i4 = 0; i4 < DK; i4 += 4) {
+                    const float4 k4 = *reinterpret_cast<const float4 *>(kq + i4), q4 = *reinterpret_cast<const float4 *>(qq + i4);
+                    S[i4] = fmaf(dconst, S[i4], k4.x * vt); o = fmaf(S[i4], q4.x, o);
+                    S[i4 + 1] = fmaf(dconst, S[i4 + 1], k4.y * vt); o = fmaf(S[i4 + 1], q4.y, o);
+                    S[i4 + 2] = fmaf(dconst, S[i4 + 2], k4.z * vt); o = fmaf(S[i4 + 2], q4.z, o);
+                    S[i4 + 3] = fmaf(dconst, S[i4 + 3], k4.w * vt); o = fmaf(S[i4 + 3], q4.w, o);
+                }
+            } else {
+                const float gt = gs[buf][tt], bt = bs[buf][tt];
+                float r = 0.0f;
+#pragma unroll
+                for (int i4 = 0; i4 < DK; i4 += 4) {
+                    const float4 k4 = *reinterpret_cast<const float4 *>(kq + i4);
+                    S[i4] *= gt; r = fmaf(S[i4], k4.x, r);
+                    S[i4 + 1] *= gt; r = fmaf(S[i4 + 1], k4.y, r);
+                    S[i4 + 2] *= gt; r = fmaf(S[i4 + 2], k4.z, r);
+                    S[i4 + 3] *= gt; r = fmaf(S[i4 + 3], k4.w, r);
+                }
+                const float u = bt * (vt - r);
+#pragma unroll
+                for (int i4 = 0; i4 < DK; i4 += 4) {
+                    const float4 k4 = *reinterpret_cast<const float4 *>(kq + i4), q4 = *reinterpret_cast<const float4 *>(qq + i4);
+                    S[i4] = fmaf(k4.x, u, S[i4]); o = fmaf(S[i4], q4.x, o);
+                    S[i4 + 1] = fmaf(k4.y, u, S[i4 + 1]); o = fmaf(S[i4 + 1], q4.y, o);
+                    S[i4 + 2] = fmaf(k4.z, u, S[i4 + 2]); o = fmaf(S[i4 + 2], q4.z, o);
+                    S[i4 + 3] = fmaf(k4.w, u, S[i4 + 3]); o = fmaf(S[i4 + 3], q4.w, o);
+                }
             }
-        } else {
-            float r = 0.0f;
-#pragma unroll
-            for (int i4 = 0; i4 < DK; i4 += 4) {
-                const float4 k4 = *reinterpret_cast<const float4 *>(ks + i4);
-                S[i4] *= gt; r = fmaf(S[i4], k4.x, r);
-                S[i4 + 1] *= gt; r = fmaf(S[i4 + 1], k4.y, r);
-                S[i4 + 2] *= gt; r = fmaf(S[i4 + 2], k4.z, r);
-                S[i4 + 3] *= gt; r = fmaf(S[i4 + 3], k4.w, r);
-            }
-            const float u = bt * (vt - r);
-#pragma unroll
-            for (int i4 = 0; i4 < DK; i4 += 4) {
-                const float4 k4 = *reinterpret_cast<const float4 *>(ks + i4), q4 = *reinterpret_cast<const float4 *>(qs + i4);
-                S[i4] = fmaf(k4.x, u, S[i4]); o = fmaf(S[i4], q4.x, o);
-                S[i4 + 1] = fmaf(k4.y, u, S[i4 + 1]); o = fmaf(S[i4 + 1], q4.y, o);
-                S[i4 + 2] = fmaf(k4.z, u, S[i4 + 2]); o = fmaf(S[i4 + 2], q4.z, o);
-                S[i4 + 3] = fmaf(k4.w, u, S[i4 + 3]); o = fmaf(S[i4 + 3], q4.w, o);
-            }
+            if (live) P.out[(size_t)(sd.row0 + t0 + tt) * P.ldo + (size_t)h * P.dv + j] = o;
         }
-        if (live) P.out[(size_t)(sd.row0 + t) * P.ldo + (size_t)h * P.dv + j] = o;
+        if (more) publish(buf ^ 1);     // (the other buffer was last read one group ago, before the barrier below)
+        __syncthreads();
     }
     if (live) {
 #pragma unroll

@@ -142,7 +142,7 @@ def test_short_convolution_with_carried_tail(taps):
 
 
 @pytest.mark.parametrize("kind", [0, 1])
-@pytest.mark.parametrize("heads,qk_heads,dk,dv", [(2, 2, 8, 8), (4, 2, 24, 70), (3, 1, 130, 33)])
+@pytest.mark.parametrize("heads,qk_heads,dk,dv", [(2, 2, 8, 8), (4, 2, 24, 70), (3, 1, 130, 33), (2, 1, 32, 40), (4, 2, 64, 64), (2, 2, 128, 100)])
 def test_state_recurrences(kind, heads, qk_heads, dk, dv):
     if kind == 0:
         qk_heads = heads
@@ -205,7 +205,7 @@ def test_delta_gates_and_gated_group_norm():
 
 @pytest.mark.parametrize("tile_min", [16, 1 << 30])       # prompts through the tiled matrix-core kernel / every row through the per-row kernel
 @pytest.mark.parametrize("heads,kv_heads,dim,window,keep,nb,dmax", [(4, 2, 16, 9, 2, 8, 30), (2, 2, 8, 1, 0, 4, 6), (3, 1, 68, 300, 5, 32, 240), (6, 3, 32, 17, 40, 10, 12),
-                                                                    (2, 1, 64, 20, 3, 8, 30), (2, 2, 128, 50, 0, 16, 100), (1, 1, 96, 9, 2, 8, 30), (4, 2, 64, 33, 33, 6, 7)])
+                                                                    (2, 1, 64, 20, 3, 8, 30), (2, 1, 32, 2000, 4, 8, 30), (2, 2, 128, 50, 0, 16, 100), (1, 1, 96, 9, 2, 8, 30), (4, 2, 64, 33, 33, 6, 7)])
 def test_windowed_attention_with_sink_cap_and_bucket_bias(heads, kv_heads, dim, window, keep, nb, dmax, tile_min):
     rng = np.random.default_rng(heads + dim + window)
     L, eps, scale, cap = 150, 1e-6, 0.3, 6.0
@@ -222,6 +222,7 @@ def test_windowed_attention_with_sink_cap_and_bucket_bias(heads, kv_heads, dim, 
     bucket_of = devi([orc.distance_bucket(n, nb, dmax) for n in range(ctx)])
     kvd = kv_heads * dim
     sl = Slots(2, 2 * ctx * kvd)
+    ws = torch.full((2 * heads * 16 * (dim + 2),), float('nan'), dtype=torch.float32, device='cuda')      # single tokens: the keys shared out over workgroups
     at = 0
     for n in (1, 2, 60, 1, 1, 80, 5):                # prompt portions and single tokens; the same sequence lives on slot 1
         d, rs, T = seq_tables([(n, at, 1)])
@@ -230,7 +231,7 @@ def test_windowed_attention_with_sink_cap_and_bucket_bias(heads, kv_heads, dim, 
         out = torch.empty((T, heads * dim), dtype=torch.float32, device="cuda")
         ia.check(capi().ifa_attention_window_f32(p(dev32(q[at:at + n])), heads * dim + 4, heads, kv_heads, dim, 1, eps, scale, cap, window, keep, p(devbf(rel)),
                                                  p(bucket_of), nb, p(devbf(sink)), p(d), p(rs), T, p(sl.table), 0, ctx * kvd, p(out), heads * dim,
-                                                 (C.c_int * 4)(0, n, at, 1), 1, tile_min, stream()))
+                                                 (C.c_int * 4)(0, n, at, 1), 1, tile_min, p(ws) if n <= 2 else None, ws.numel() * 4, stream()))
         sync()
         assert np.abs(out.cpu().numpy() - want[at:at + n]).max() < 2e-5 * max(1.0, np.abs(want).max()), (at, n)
         at += n
@@ -239,7 +240,7 @@ def test_windowed_attention_with_sink_cap_and_bucket_bias(heads, kv_heads, dim, 
     d, rs, T = seq_tables([(1, L - 1, 1)])
     out = torch.empty((1, heads * dim), dtype=torch.float32, device="cuda")
     ia.check(capi().ifa_attention_window_f32(p(dev32(q[L - 1:])), heads * dim + 4, heads, kv_heads, dim, 1, eps, scale, cap, window, keep, p(devbf(rel)),
-                                             p(bucket_of), nb, None, p(d), p(rs), T, p(sl.table), 0, ctx * kvd, p(out), heads * dim, None, 0, 0, stream()))
+                                             p(bucket_of), nb, None, p(d), p(rs), T, p(sl.table), 0, ctx * kvd, p(out), heads * dim, None, 0, 0, None, 0, stream()))
     assert np.abs(out.cpu().numpy() - want[L - 1:]).max() > 1e-4
 
 
@@ -267,7 +268,7 @@ def test_windowed_attention_tiles_over_several_sequences():
             host += [r, n, pos0, slot]; r += n
         ia.check(capi().ifa_attention_window_f32(p(qd), heads * dim, heads, kv_heads, dim, 1, eps, scale, cap, window, keep, p(devbf(rel)), p(bucket_of), nb,
                                                  p(devbf(sink)), p(d), p(rs), T, p(sl.table), 0, ctx * kvd, p(out), heads * dim, (C.c_int * len(host))(*host),
-                                                 len(seqs), 16, stream()))
+                                                 len(seqs), 16, None, 0, stream()))
         sync()
         got, r = out.cpu().numpy(), 0
         for s_, n in step:
