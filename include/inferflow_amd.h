@@ -458,9 +458,11 @@ int ifa_model_time_kernel(ifa_model *m, int which, int iters, float *avg_us);
 /* C[t][n] (+)= alpha * mul[n] * (sum_k A[t][k] W[n][k] + bias[n]);  W bf16 [rows][cols], A fp32 [tokens][lda], C fp32 [tokens][ldc];
  * bias / mul (bf16 [rows]) nullable; accumulate != 0 adds into C (the residual update of a layer).  ops32 != 0 keeps the operands
  * of the matrix-core product in fp32 (v_mfma_f32_32x32x2_f32) instead of rounding them to bfloat16; up to 8 tokens the product is
- * a weight-streaming fp32 dot either way.  fp32 accumulation, no atomics: deterministic. */
+ * a weight-streaming fp32 dot either way.  Output columns [silu_col0, silu_col1) pass SiLU right after the bias (empty range: none).
+ * fp32 accumulation, no atomics: deterministic. */
 int ifa_linear_bf16w(const void *w_bf16, size_t rows, size_t cols, const void *a_f32, size_t lda, size_t tokens, const void *bias_bf16,
-                     const void *mul_bf16, float alpha, int accumulate, int ops32, void *c_f32, size_t ldc, ifa_stream stream);
+                     const void *mul_bf16, float alpha, int accumulate, int ops32, void *c_f32, size_t ldc, int silu_col0, int silu_col1,
+                     ifa_stream stream);
 /* x[t] = embed[token_t] + pe(pos_t), pe[2i] = sin(p base^(-2i/width)), pe[2i+1] = cos(same); angles formed in double */
 int ifa_embed_sinpos_f32(const void *embed_bf16, int vocab, int width, const int *tokens_dev, const int *positions_dev, size_t tokens,
                          float base, void *x_f32, ifa_stream stream);

@@ -191,9 +191,9 @@ int ensure_logits(ifa_model *m, size_t rows)
 }
 
 int linear(ifa_model *m, const bf16_t *W, size_t N, size_t K, const float *A, size_t lda, size_t T, const bf16_t *bias, const bf16_t *mul, float alpha,
-           int accumulate, float *C, size_t ldc)
+           int accumulate, float *C, size_t ldc, int silu0 = 0, int silu1 = 0)
 {
-    return ifa_linear_bf16w(W, N, K, A, lda, T, bias, mul, alpha, accumulate, m->lay->cfg.ops32, C, ldc, (ifa_stream)m->stream);
+    return ifa_linear_bf16w(W, N, K, A, lda, T, bias, mul, alpha, accumulate, m->lay->cfg.ops32, C, ldc, silu0, silu1, (ifa_stream)m->stream);
 }
 
 // the layers of one step over T rows / nseq sequences whose tables are already on the device; leaves the residual in n->x
@@ -212,7 +212,9 @@ int run_layers(ifa_model *m, size_t T, int nseq)
         const bf16_t *ls1 = (const bf16_t *)L.T(IFA_LT_LS1).data;
         if ((rc = ifa_layernorm_f32(1, n->x, W, T, W, L.T(IFA_LT_NORM1).data, c.eps, n->h, W, s))) return rc;
         const size_t NI = L.n_in;
-        if ((rc = linear(m, L.w_in, NI, W, n->h, W, T, L.b_in, nullptr, 1.0f, 0, n->proj, NI))) return rc;
+        // (the linear attention's q | k | v leave the product through SiLU: contiguous columns [c_lq, c_lg))
+        const bool lin = sp.mixer == IFA_MIX_WINDOW_LINEAR;
+        if ((rc = linear(m, L.w_in, NI, W, n->h, W, T, L.b_in, nullptr, 1.0f, 0, n->proj, NI, lin ? (int)L.c_lq : 0, lin ? (int)L.c_lg : 0))) return rc;
         if (sp.mixer == IFA_MIX_WINDOW_LINEAR) {
             const size_t AQ = (size_t)sp.a_heads * sp.a_dim, LV = (size_t)sp.l_heads * sp.l_vdim;
             // windowed attention: the values are the keys as projected; the cache's K rows hold the normed keys
@@ -223,7 +225,7 @@ int run_layers(ifa_model *m, size_t T, int nseq)
                                                n->row_seq_dev, T, slots, L.o_k, L.o_v, n->m1, AQ, n->seqs_host.data(), (int)n->seqs_host.size(), n->opt_attn_tile_min, n->attn_ws, n->attn_ws_bytes, s))) return rc;
             if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_A_O).data, W, AQ, n->m1, AQ, T, nullptr, ls1, sp.a_out_scale, 1, n->x, W))) return rc;
             // decayed linear attention
-            if ((rc = ifa_state_scan_f32(0, 1, n->proj + L.c_lq, NI, n->proj + L.c_lk, NI, n->proj + L.c_lv, NI, sp.l_heads, sp.l_heads, sp.l_dim, sp.l_vdim,
+            if ((rc = ifa_state_scan_f32(0, 0, n->proj + L.c_lq, NI, n->proj + L.c_lk, NI, n->proj + L.c_lv, NI, sp.l_heads, sp.l_heads, sp.l_dim, sp.l_vdim,
                                          L.T(IFA_LT_L_DECAY).data, nullptr, nullptr, n->seqs_dev, nseq, slots, L.o_lin, n->m2, LV, s))) return rc;
             if ((rc = ifa_gated_groupnorm_f32(n->m2, LV, T, (int)LV, (int)LV, L.T(IFA_LT_L_NORM).data, (int)LV, n->proj + L.c_lg, NI, 0, c.eps, n->m2, LV, s))) return rc;
             if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_L_O).data, W, LV, n->m2, LV, T, nullptr, ls1, sp.l_out_scale, 1, n->x, W))) return rc;

@@ -1,5 +1,6 @@
 // ifa_linear_bf16.hip -- linear layers with bfloat16 weights [N][K] and 32-bit activations [T][K]:
-//   C[t][n] (+)= alpha * mul[n] * (sum_k A[t][k] W[n][k] + bias[n])        (mul, bias optional; C in 32-bit floats)
+//   C[t][n] (+)= alpha * mul[n] * act(sum_k A[t][k] W[n][k] + bias[n])     (mul, bias optional; act = SiLU on a column range, else identity;
+//                                                                          C in 32-bit floats)
 // The epilogue covers a plain projection (store), a projection with bias, and the residual update of a layer
 // (accumulate into the 32-bit residual stream with a per-channel layer scale and a branch scale).
 //
@@ -25,11 +26,13 @@ struct LinArgs {
     const bf16_t *bias, *mul;
     int T, N, K, lda, ldc;
     float alpha; int accumulate, vec;
+    int act_c0, act_c1;          // output columns [act_c0, act_c1) pass SiLU after the bias (projections whose consumer wants them activated)
 };
 
 __device__ __forceinline__ void lin_store(const LinArgs &P, int t, int n, float acc)
 {
     if (P.bias) acc += bf2f(P.bias[n]);
+    if (n >= P.act_c0 && n < P.act_c1) acc = silu_exact(acc);
     if (P.mul) acc *= bf2f(P.mul[n]);
     acc *= P.alpha;
     float *c = P.C + (size_t)t * P.ldc + n;
@@ -172,7 +175,7 @@ __global__ void __launch_bounds__(256) k_lin_rows(LinArgs P)
 
 extern "C" int ifa_linear_bf16w(const void *w_bf16, size_t rows, size_t cols, const void *a_f32, size_t lda, size_t tokens,
                                 const void *bias_bf16, const void *mul_bf16, float alpha, int accumulate, int ops32,
-                                void *c_f32, size_t ldc, ifa_stream stream)
+                                void *c_f32, size_t ldc, int silu_col0, int silu_col1, ifa_stream stream)
 {
     IFA_REQUIRE(w_bf16 && a_f32 && c_f32, "ifa_linear_bf16w: null pointer");
     IFA_REQUIRE(rows > 0 && cols > 0 && tokens > 0 && lda >= cols && ldc >= rows, "ifa_linear_bf16w: bad shape (%zu x %zu, %zu tokens, lda %zu, ldc %zu)", rows, cols, tokens, lda, ldc);
@@ -181,7 +184,7 @@ extern "C" int ifa_linear_bf16w(const void *w_bf16, size_t rows, size_t cols, co
     P.W = (const bf16_t *)w_bf16; P.A = (const float *)a_f32; P.C = (float *)c_f32;
     P.bias = (const bf16_t *)bias_bf16; P.mul = (const bf16_t *)mul_bf16;
     P.T = (int)tokens; P.N = (int)rows; P.K = (int)cols; P.lda = (int)lda; P.ldc = (int)ldc;
-    P.alpha = alpha; P.accumulate = accumulate ? 1 : 0;
+    P.alpha = alpha; P.accumulate = accumulate ? 1 : 0; P.act_c0 = silu_col0; P.act_c1 = silu_col1;
     // 16-byte requests need whole 8-element pieces in every row of both operands
     P.vec = (cols % 8 == 0 && lda % 4 == 0 && ((uintptr_t)a_f32 & 15) == 0 && ((uintptr_t)w_bf16 & 15) == 0) ? 1 : 0;
     hipStream_t s = ifa_s(stream);

@@ -162,32 +162,42 @@ __global__ void __launch_bounds__(64) k_state_scan(ScanArgs P)
     if (live) for (int i = 0; i < dk; i++) state[(size_t)i * P.dv + j] = S[i * 64 + lane];
 }
 
-// The same recurrences with the column S[:, j] of a lane in REGISTERS (key sizes 32 / 64 / 128).  Tokens go in groups of 8: the
-// group's q, k (and gates) sit in LDS and are broadcast in 16-byte reads, the NEXT group's operands are requested from memory before
-// the current group is computed (a token is ~0.3 us of dependent arithmetic; a memory round trip is longer than that).  A token costs
-// DK / 2 LDS reads and 2 DK (decay) or 3 DK (delta rule) fp32 operations per lane.  Same order of operations per element as the
-// general kernel above: bit-identical results.
+// The same recurrences for key sizes 32 / 64 / 128 with the state in REGISTERS and FOUR lanes per column: lane 4 c + r of a wave owns
+// rows [r DK / 4, (r + 1) DK / 4) of column c (16 columns per wave), so a token is DK / 4 elements of dependent arithmetic per lane
+// instead of DK -- the recurrence is a chain of dependent instructions of a wave that is alone on its SIMD, and its length per token
+// is what the prompt rate of these layers comes down to.  The sums over a column's rows (the read-out, and S^T k of the delta rule)
+// are finished across the four lanes by two DPP quad permutes.  Tokens go in groups of 8: the group's q, k and gates are staged in
+// LDS (16-byte reads of a lane's row range), the next group's operands are requested from memory before the current group is
+// computed.  fp32 results differ from the general kernel's by the order of these sums only.
 constexpr int SCAN_TB = 8;
+
+__device__ __forceinline__ float quad_sum(float v)
+{
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));      // lanes ^ 1
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));      // lanes ^ 2
+    return v;
+}
 
 template <int KIND, int DK>
 __global__ void __launch_bounds__(64) k_state_scan_reg(ScanArgs P)
 {
+    constexpr int DKQ = DK / 4;
     __shared__ __attribute__((aligned(16))) float qs[2][SCAN_TB][DK], ks[2][SCAN_TB][DK];
     __shared__ float gs[2][SCAN_TB], bs[2][SCAN_TB];
     const int seq = blockIdx.x / P.heads, h = blockIdx.x % P.heads;
-    const int lane = threadIdx.x, j = blockIdx.y * 64 + lane;
+    const int lane = threadIdx.x, rg = lane & 3, j = blockIdx.y * 16 + (lane >> 2);
     const bool live = j < P.dv;
     const int jc = live ? j : P.dv - 1;
     const int qh = h / (P.heads / P.qk_heads);
     const SeqDesc sd = P.seqs[seq];
-    float *state = P.slot_base[sd.slot] + P.state_off + (size_t)h * DK * P.dv;
-    float S[DK];
+    float *state = P.slot_base[sd.slot] + P.state_off + ((size_t)h * DK + (size_t)rg * DKQ) * P.dv;
+    float S[DKQ];
     if (sd.pos0 > 0) {
 #pragma unroll
-        for (int i = 0; i < DK; i++) S[i] = state[(size_t)i * P.dv + jc];
+        for (int e = 0; e < DKQ; e++) S[e] = state[(size_t)e * P.dv + jc];
     } else {
 #pragma unroll
-        for (int i = 0; i < DK; i++) S[i] = 0.0f;
+        for (int e = 0; e < DKQ; e++) S[e] = 0.0f;
     }
     const float dconst = KIND == 0 ? P.decay_head[h] : 0.0f;
     constexpr int PER = SCAN_TB * DK / 64;          // q (and k) values of a group per lane
@@ -224,48 +234,49 @@ __global__ void __launch_bounds__(64) k_state_scan_reg(ScanArgs P)
         const bool more = t0 + SCAN_TB < sd.n;
         if (more) request(t0 + SCAN_TB);
         const int cnt = min(SCAN_TB, sd.n - t0);
-        for (int tt = 0; tt < cnt; tt++) {
-            const float vt = vcur[tt];
-            const float *kq = ks[buf][tt], *qq = qs[buf][tt];
-            float o = 0.0f;
-            if (KIND == 0) {
 #pragma unroll
-                for (int i4 = 0; i4 < DK; i4 += 4) {
-                    const float4 k4 = *reinterpret_cast<const float4 *>(kq + i4), q4 = *reinterpret_cast<const float4 *>(qq + i4);
-                    S[i4] = fmaf(dconst, S[i4], k4.x * vt); o = fmaf(S[i4], q4.x, o);
-                    S[i4 + 1] = fmaf(dconst, S[i4 + 1], k4.y * vt); o = fmaf(S[i4 + 1], q4.y, o);
-                    S[i4 + 2] = fmaf(dconst, S[i4 + 2], k4.z * vt); o = fmaf(S[i4 + 2], q4.z, o);
-                    S[i4 + 3] = fmaf(dconst, S[i4 + 3], k4.w * vt); o = fmaf(S[i4 + 3], q4.w, o);
-                }
-            } else {
-                const float gt = gs[buf][tt], bt = bs[buf][tt];
-                float r = 0.0f;
+        for (int tt = 0; tt < SCAN_TB; tt++) {
+            if (tt < cnt) {
+                const float vt = vcur[tt];
+                float kk[DKQ], qq[DKQ];
 #pragma unroll
-                for (int i4 = 0; i4 < DK; i4 += 4) {
-                    const float4 k4 = *reinterpret_cast<const float4 *>(kq + i4);
-                    S[i4] *= gt; r = fmaf(S[i4], k4.x, r);
-                    S[i4 + 1] *= gt; r = fmaf(S[i4 + 1], k4.y, r);
-                    S[i4 + 2] *= gt; r = fmaf(S[i4 + 2], k4.z, r);
-                    S[i4 + 3] *= gt; r = fmaf(S[i4 + 3], k4.w, r);
+                for (int e4 = 0; e4 < DKQ; e4 += 4) {
+                    const float4 k4 = *reinterpret_cast<const float4 *>(&ks[buf][tt][rg * DKQ + e4]), q4 = *reinterpret_cast<const float4 *>(&qs[buf][tt][rg * DKQ + e4]);
+                    kk[e4] = k4.x; kk[e4 + 1] = k4.y; kk[e4 + 2] = k4.z; kk[e4 + 3] = k4.w;
+                    qq[e4] = q4.x; qq[e4 + 1] = q4.y; qq[e4 + 2] = q4.z; qq[e4 + 3] = q4.w;
                 }
-                const float u = bt * (vt - r);
+                float o0 = 0.0f, o1 = 0.0f;
+                if (KIND == 0) {
 #pragma unroll
-                for (int i4 = 0; i4 < DK; i4 += 4) {
-                    const float4 k4 = *reinterpret_cast<const float4 *>(kq + i4), q4 = *reinterpret_cast<const float4 *>(qq + i4);
-                    S[i4] = fmaf(k4.x, u, S[i4]); o = fmaf(S[i4], q4.x, o);
-                    S[i4 + 1] = fmaf(k4.y, u, S[i4 + 1]); o = fmaf(S[i4 + 1], q4.y, o);
-                    S[i4 + 2] = fmaf(k4.z, u, S[i4 + 2]); o = fmaf(S[i4 + 2], q4.z, o);
-                    S[i4 + 3] = fmaf(k4.w, u, S[i4 + 3]); o = fmaf(S[i4 + 3], q4.w, o);
+                    for (int e = 0; e < DKQ; e += 2) {
+                        S[e] = fmaf(dconst, S[e], kk[e] * vt); o0 = fmaf(S[e], qq[e], o0);
+                        S[e + 1] = fmaf(dconst, S[e + 1], kk[e + 1] * vt); o1 = fmaf(S[e + 1], qq[e + 1], o1);
+                    }
+                } else {
+                    const float gt = gs[buf][tt], bt = bs[buf][tt];
+                    float r0 = 0.0f, r1 = 0.0f;
+#pragma unroll
+                    for (int e = 0; e < DKQ; e += 2) {
+                        S[e] *= gt; r0 = fmaf(S[e], kk[e], r0);
+                        S[e + 1] *= gt; r1 = fmaf(S[e + 1], kk[e + 1], r1);
+                    }
+                    const float u = bt * (vt - quad_sum(r0 + r1));
+#pragma unroll
+                    for (int e = 0; e < DKQ; e += 2) {
+                        S[e] = fmaf(kk[e], u, S[e]); o0 = fmaf(S[e], qq[e], o0);
+                        S[e + 1] = fmaf(kk[e + 1], u, S[e + 1]); o1 = fmaf(S[e + 1], qq[e + 1], o1);
+                    }
                 }
+                const float o = quad_sum(o0 + o1);
+                if (live && rg == 0) P.out[(size_t)(sd.row0 + t0 + tt) * P.ldo + (size_t)h * P.dv + j] = o;
             }
-            if (live) P.out[(size_t)(sd.row0 + t0 + tt) * P.ldo + (size_t)h * P.dv + j] = o;
         }
         if (more) publish(buf ^ 1);     // (the other buffer was last read one group ago, before the barrier below)
         __syncthreads();
     }
     if (live) {
 #pragma unroll
-        for (int i = 0; i < DK; i++) state[(size_t)i * P.dv + j] = S[i];
+        for (int e = 0; e < DKQ; e++) state[(size_t)e * P.dv + j] = S[e];
     }
 }
 
@@ -351,14 +362,15 @@ int ifa_state_scan_f32(int kind, int in_act, const void *q_f32, size_t ldq, cons
     P.out = (float *)out_f32; P.ldo = ldo;
     const size_t smem = ((size_t)dk * 64 + 2 * (size_t)dk) * 4;
     const dim3 grid((unsigned)(n_seqs * heads), ifa_cdiv((size_t)dv, 64));
+    const dim3 grid16((unsigned)(n_seqs * heads), ifa_cdiv((size_t)dv, 16));
 #define IFA_SCAN_REG(DKV) \
     if (dk == DKV) { \
-        if (kind == 0) hipLaunchKernelGGL((k_state_scan_reg<0, DKV>), grid, dim3(64), 0, ifa_s(stream), P); \
-        else hipLaunchKernelGGL((k_state_scan_reg<1, DKV>), grid, dim3(64), 0, ifa_s(stream), P); \
+        if (kind == 0) hipLaunchKernelGGL((k_state_scan_reg<0, DKV>), grid16, dim3(64), 0, ifa_s(stream), P); \
+        else hipLaunchKernelGGL((k_state_scan_reg<1, DKV>), grid16, dim3(64), 0, ifa_s(stream), P); \
         IFA_LAUNCH_CHECK(); \
         return IFA_OK; \
     }
-    IFA_SCAN_REG(32) IFA_SCAN_REG(64) IFA_SCAN_REG(128)
+    IFA_SCAN_REG(16) IFA_SCAN_REG(32) IFA_SCAN_REG(64) IFA_SCAN_REG(128)
 #undef IFA_SCAN_REG
     if (kind == 0) {
         IFA_HIP_CHECK(hipFuncSetAttribute((const void *)k_state_scan<0>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));

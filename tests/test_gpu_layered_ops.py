@@ -60,9 +60,11 @@ def test_linear_bf16_weights(T, N, K):
         for use_bias, use_mul, alpha, acc in ((0, 0, 1.0, 0), (1, 0, 1.0, 0), (1, 1, 0.7, 1), (0, 1, 1.3, 1)):
             c = dev32(C0)
             ia.check(capi().ifa_linear_bf16w(p(devbf(W)), N, K, p(dev32(A)), K + 4, T, p(devbf(bias)) if use_bias else None,
-                                             p(devbf(mul)) if use_mul else None, alpha, acc, ops32, p(c), N + 2, stream()))
+                                             p(devbf(mul)) if use_mul else None, alpha, acc, ops32, p(c), N + 2, 2, min(N, 40) if use_mul else 0, stream()))
             sync()
             want = prod + (bias if use_bias else 0)
+            if use_mul:                                                 # columns [2, 40) through SiLU after the bias
+                want[:, 2:min(N, 40)] = orc.silu(orc.t64(want[:, 2:min(N, 40)])).numpy()
             if use_mul:
                 want = want * mul
             want = want * alpha + (C0[:, :N] if acc else 0)
@@ -142,7 +144,7 @@ def test_short_convolution_with_carried_tail(taps):
 
 
 @pytest.mark.parametrize("kind", [0, 1])
-@pytest.mark.parametrize("heads,qk_heads,dk,dv", [(2, 2, 8, 8), (4, 2, 24, 70), (3, 1, 130, 33), (2, 1, 32, 40), (4, 2, 64, 64), (2, 2, 128, 100)])
+@pytest.mark.parametrize("heads,qk_heads,dk,dv", [(2, 2, 8, 8), (4, 2, 24, 70), (3, 1, 130, 33), (2, 1, 32, 40), (4, 2, 64, 64), (2, 2, 128, 100), (2, 1, 16, 17)])
 def test_state_recurrences(kind, heads, qk_heads, dk, dv):
     if kind == 0:
         qk_heads = heads
