@@ -159,5 +159,56 @@ def build_library(force=False, verbose=False, jobs=None):
     return LIB_PATH
 
 
+# ---- profile "layered": a library with the layer-list worker class only (what bin/trace_run builds in a fresh checkout)
+LAYERED_LIB_PATH = os.path.join(LIB_DIR, "libinferflow_amd_layered.so")
+LAYERED_CLI_PATH = os.path.join(BIN_DIR, "ifa_trace_run_layered")
+LAYERED_UNITS = ["ifa_runtime.hip", "ifa_linear_bf16.hip", "ifa_ops_f32.hip", "ifa_seqmix.hip", "ifa_attn_window.hip", "ifa_engine_layered.hip",
+                 os.path.join("profile_layered", "ifa_model_api.hip")]
+
+
+def layered_is_stale():
+    if not (os.path.exists(LAYERED_LIB_PATH) and os.path.exists(LAYERED_CLI_PATH)):
+        return True
+    t = min(os.path.getmtime(LAYERED_LIB_PATH), os.path.getmtime(LAYERED_CLI_PATH))
+    deps = [os.path.join(CSRC, u) for u in LAYERED_UNITS] + glob.glob(os.path.join(CSRC, "*.h")) + glob.glob(os.path.join(_HERE, "..", "include", "*.h"))
+    deps += glob.glob(os.path.join(HOST, "*.cc")) + glob.glob(os.path.join(HOST, "*.h"))
+    return any(os.path.getmtime(d) > t for d in deps)
+
+
+def build_layered_library(force=False):
+    """libinferflow_amd_layered.so + bin/ifa_trace_run_layered: seven HIP units and the host engine (seconds, not minutes)."""
+    if not force and not layered_is_stale():
+        return LAYERED_LIB_PATH
+    hipcc = _hipcc()
+    if hipcc is None:
+        raise RuntimeError("hipcc not found: cannot build libinferflow_amd_layered.so")
+    obj_dir = os.path.join(LIB_DIR, "obj_layered")
+    os.makedirs(obj_dir, exist_ok=True)
+    os.makedirs(BIN_DIR, exist_ok=True)
+    inc = os.path.join(_HERE, "..", "include")
+    cxx = shutil.which("g++") or hipcc
+    procs, objs = [], []
+    for u in LAYERED_UNITS:
+        obj = os.path.join(obj_dir, os.path.basename(u) + ".o")
+        objs.append(obj)
+        procs.append((u, subprocess.Popen([hipcc] + HIPCC_FLAGS + ["-I", inc, "-I", CSRC, "-c", os.path.join(CSRC, u), "-o", obj],
+                                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
+    for src in host_sources():
+        obj = os.path.join(obj_dir, "host_" + os.path.basename(src) + ".o")
+        objs.append(obj)
+        procs.append((src, subprocess.Popen([cxx] + HOST_FLAGS + ["-I", inc, "-I", HOST, "-c", src, "-o", obj], stdout=subprocess.PIPE, stderr=subprocess.STDOUT)))
+    failed = []
+    for src, p in procs:
+        out, _ = p.communicate()
+        if p.returncode != 0:
+            failed.append((src, out.decode(errors="replace")))
+    if failed:
+        raise RuntimeError("build failed:\n" + "\n".join("== %s ==\n%s" % f for f in failed))
+    subprocess.check_call([hipcc, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", LAYERED_LIB_PATH] + objs)
+    subprocess.check_call([cxx] + HOST_FLAGS + ["-I", inc, "-I", HOST, os.path.join(HOST, "trace_run_main.cc"), "-o", LAYERED_CLI_PATH,
+                           "-L", LIB_DIR, "-linferflow_amd_layered", "-Wl,-rpath,$ORIGIN/../lib"])
+    return LAYERED_LIB_PATH
+
+
 if __name__ == "__main__":
     print(build_library(force="--force" in sys.argv, verbose=True))

@@ -49,8 +49,8 @@ struct WinAttnArgs {
 
 constexpr int WA_DPL = 4;         // dim <= 64 * WA_DPL
 
-// grid (rows, heads), four waves: the visible keys (kept first tokens, then the window) are walked in chunks of 64, one
-// key per lane for the score, one value column per lane for the weighted sum; chunks go round-robin to the waves, each
+// grid (rows, heads, splits), four waves: the visible keys (kept first tokens, then the window) are walked in chunks of 16, four
+// lanes per key for the score, one value column per lane for the weighted sum; chunks go round-robin to the waves, each
 // with its own running maximum / sum / accumulator, merged through LDS at the end together with the sink.
 __global__ void __launch_bounds__(256) k_attn_window(WinAttnArgs P)
 {
@@ -77,37 +77,38 @@ __global__ void __launch_bounds__(256) k_attn_window(WinAttnArgs P)
     float m = -INFINITY, l = 0.0f, acc[WA_DPL];
 #pragma unroll
     for (int e = 0; e < WA_DPL; e++) acc[e] = 0.0f;
-    const int nchunks = (nk + 63) / 64;
+    // 16 keys per wave and step, four lanes per key (each a quarter of the dot product in interleaved 16-byte pieces, finished by a quad sum)
+    const int nchunks = (nk + 15) / 16, sub = lane & 3;
     const int nsplit = max(1, P.nsplit), split = blockIdx.z;
     for (int ch = split * 4 + wave; ch < nchunks; ch += 4 * nsplit) {
-        const int vi = ch * 64 + lane;
+        const int vi = ch * 16 + (lane >> 2);
         const bool valid = vi < nk;
         const int j = valid ? (vi < nkeep ? vi : lo + (vi - nkeep)) : i;
         const float *kr = kc + (size_t)j * kvd;
         float s = 0.0f;
         if ((dim & 3) == 0) {
-            for (int c = 0; c < dim; c += 4) {
+            for (int c = 4 * sub; c < dim; c += 16) {
                 const float4 kv = *reinterpret_cast<const float4 *>(kr + c);
                 s = fmaf(qn[c], kv.x, s); s = fmaf(qn[c + 1], kv.y, s); s = fmaf(qn[c + 2], kv.z, s); s = fmaf(qn[c + 3], kv.w, s);
             }
         } else {
-            for (int c = 0; c < dim; c++) s = fmaf(qn[c], kr[c], s);
+            for (int c = sub; c < dim; c += 4) s = fmaf(qn[c], kr[c], s);
         }
-        s *= P.scale;
+        s = quad_sum(s) * P.scale;
         if (P.softcap > 0.0f) s = P.softcap * tanhf(s / P.softcap);
         if (P.rel) s += bf2f(P.rel[(size_t)P.bucket_of[i - j] * P.heads + h]);
         if (!valid) s = -INFINITY;
         const float m_new = fmaxf(m, wave_max(s));          // finite: the chunk holds at least one visible key
         const float p = valid ? expf(s - m_new) : 0.0f;
         const float corr = m == -INFINITY ? 0.0f : expf(m - m_new);
-        l = l * corr + wave_sum(p);
+        l = l * corr + wave_sum(sub == 0 ? p : 0.0f);
 #pragma unroll
         for (int e = 0; e < WA_DPL; e++) acc[e] *= corr;
         m = m_new;
-        const int cnt = min(64, nk - ch * 64);
+        const int cnt = min(16, nk - ch * 16);
         for (int jj = 0; jj < cnt; jj++) {
-            const float pj = __shfl(p, jj, 64);
-            const int kj = __shfl(j, jj, 64);
+            const float pj = __shfl(p, 4 * jj, 64);
+            const int kj = __shfl(j, 4 * jj, 64);
             const float *vr = vc + (size_t)kj * kvd;
 #pragma unroll
             for (int e = 0; e < WA_DPL; e++) { const int d = lane + 64 * e; if (d < dim) acc[e] = fmaf(pj, vr[d], acc[e]); }
@@ -348,7 +349,7 @@ int ifa_attention_window_f32(const void *q_f32, size_t ldq, int heads, int kv_he
     // few rows: a (row, head)'s keys are shared out to several workgroups (one workgroup pulls its keys through ONE compute unit)
     int nsplit = 1;
     if (ws_f32 && rows * (size_t)heads <= 512) {
-        nsplit = (int)std::min<size_t>(16, ((size_t)window + (size_t)keep_first + 255) / 256);
+        nsplit = (int)std::min<size_t>(16, ((size_t)window + (size_t)keep_first + 127) / 128);
         while (nsplit > 1 && rows * (size_t)heads * nsplit * ((size_t)dim + 2) * 4 > ws_bytes) nsplit--;
     }
     P.ws = (float *)ws_f32; P.nsplit = nsplit;

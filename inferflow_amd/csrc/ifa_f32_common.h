@@ -39,6 +39,14 @@ __device__ __forceinline__ float wave_max(float v)
     return v;
 }
 
+// sum over the four lanes 4 q .. 4 q + 3 (two DPP quad permutes); every one of them gets the result
+__device__ __forceinline__ float quad_sum(float v)
+{
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));      // lanes ^ 1
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));      // lanes ^ 2
+    return v;
+}
+
 // sum over a workgroup of up to 1024 threads; red: 17 floats of LDS; every thread gets the result
 __device__ __forceinline__ float block_sum(float v, float *red)
 {

@@ -171,13 +171,6 @@ __global__ void __launch_bounds__(64) k_state_scan(ScanArgs P)
 // computed.  fp32 results differ from the general kernel's by the order of these sums only.
 constexpr int SCAN_TB = 8;
 
-__device__ __forceinline__ float quad_sum(float v)
-{
-    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0xB1, 0xF, 0xF, true));      // lanes ^ 1
-    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x4E, 0xF, 0xF, true));      // lanes ^ 2
-    return v;
-}
-
 template <int KIND, int DK>
 __global__ void __launch_bounds__(64) k_state_scan_reg(ScanArgs P)
 {
@@ -288,6 +281,21 @@ __global__ void __launch_bounds__(256) k_gated_groupnorm(const float *__restrict
     const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
     const float *orow = o + (size_t)t * ldo, *grow = gate + (size_t)t * ldg;
     float *yrow = y + (size_t)t * ldy;
+    if (C / group < nw) {          // fewer groups than waves (one norm over all heads): the whole workgroup works on each group
+        __shared__ float red[17];
+        for (int gi = 0; gi < C / group; gi++) {
+            float s = 0.0f;
+            for (int e = threadIdx.x; e < group; e += blockDim.x) { const float v = orow[gi * group + e]; s = fmaf(v, v, s); }
+            const float r = 1.0f / sqrtf(block_sum(s, red) / (float)group + eps);
+            for (int e = threadIdx.x; e < group; e += blockDim.x) {
+                const int c = gi * group + e;
+                const float gv = grow[c];
+                const float ga = gate_act == 0 ? sigmoid_f(gv) : silu_exact(gv);
+                yrow[c] = orow[c] * r * bf2f(w[c % wlen]) * ga;
+            }
+        }
+        return;
+    }
     for (int gi = wave; gi < C / group; gi += nw) {
         float s = 0.0f;
         for (int e = lane; e < group; e += 64) { const float v = orow[gi * group + e]; s = fmaf(v, v, s); }

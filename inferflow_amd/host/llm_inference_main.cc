@@ -2,8 +2,9 @@
 // (src/tools/llm_inference.cc:345-457): load the .ini, add one query, then loop
 // Infer -> pick the greedy token -> CommitInferenceResult, and report prefill / decode rates.
 //
-//   ifa_llm_inference <config.ini> [--section transformer_engine] [--tokens 1,15043,3186]
-//                     [--prompt-len N --seed S] [--max-new 64] [--generate]
+//   ifa_llm_inference <config.ini | model directory> [--section transformer_engine] [--tokens 1,15043,3186]
+//                     [--prompt-len N --seed S] [--max-new 64] [--generate] [--dtype bfloat16|float32 --max-ctx N]
+// A model directory (config.json naming a registered layer-list architecture + model.safetensors) needs no .ini.
 // --generate uses InferenceEngine::Generate (device-side token feedback) instead of the per-step loop.
 #include <chrono>
 #include <cstdio>
@@ -17,9 +18,9 @@ using namespace inferflow_amd;
 
 int main(int argc, char **argv)
 {
-    if (argc < 2) { fprintf(stderr, "usage: %s <config.ini> [--section S] [--tokens a,b,c] [--prompt-len N] [--seed S] [--max-new N] [--generate]\n", argv[0]); return 2; }
-    std::string ini = argv[1], section = "transformer_engine", tokens_arg;
-    int prompt_len = 16, max_new = 64; unsigned seed = 42; bool generate = false;
+    if (argc < 2) { fprintf(stderr, "usage: %s <config.ini | model dir> [--section S] [--tokens a,b,c] [--prompt-len N] [--seed S] [--max-new N] [--generate]\n", argv[0]); return 2; }
+    std::string ini = argv[1], section = "transformer_engine", tokens_arg, dtype = "bfloat16";
+    int prompt_len = 16, max_new = 64, max_ctx = 4096; unsigned seed = 42; bool generate = false;
     for (int i = 2; i < argc; i++) {
         const std::string a = argv[i];
         auto next = [&]() -> const char * { return i + 1 < argc ? argv[++i] : ""; };
@@ -29,10 +30,17 @@ int main(int argc, char **argv)
         else if (a == "--seed") seed = (unsigned)atoi(next());
         else if (a == "--max-new") max_new = atoi(next());
         else if (a == "--generate") generate = true;
+        else if (a == "--dtype") dtype = next();
+        else if (a == "--max-ctx") max_ctx = atoi(next());
         else { fprintf(stderr, "unknown option %s\n", a.c_str()); return 2; }
     }
     InferenceConfig cfg;
-    if (!InferenceEngine::LoadConfig(cfg, ini, section)) { fprintf(stderr, "LoadConfig: %s\n", EngineLastError()); return 1; }
+    // a model directory instead of an .ini: config.json with a registered layer-list architecture + model.safetensors
+    std::string arch;
+    const std::string as_dir = ini.empty() || ini.back() == '/' ? ini : ini + "/";
+    if (LayeredArchitectureOf(as_dir, arch)) {
+        if (!InferenceEngine::LoadConfigForModelDir(cfg, as_dir, dtype, max_ctx, 2)) { fprintf(stderr, "LoadConfig: %s\n", EngineLastError()); return 1; }
+    } else if (!InferenceEngine::LoadConfig(cfg, ini, section)) { fprintf(stderr, "LoadConfig: %s\n", EngineLastError()); return 1; }
     InferenceEngine engine;
     auto t0 = std::chrono::steady_clock::now();
     if (!engine.Init(cfg)) { fprintf(stderr, "Init: %s\n", EngineLastError()); return 1; }
