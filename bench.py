@@ -407,6 +407,9 @@ def run_arch_bench(args):
             eng = InferenceEngine.from_model_dir(d, "bfloat16", ctx, 2, False)
         finally:
             shutil.rmtree(d, ignore_errors=True)
+        if os.environ.get("IFA_FUSE_ROWS"):      # measurement: 0 none, 1 norm, 2 gated GELU, 3 both folded into the row products
+            import inferflow_amd as ia
+            ia.check(ia.lib().ifa_model_set_option(eng.worker(), b"fuse_rows", int(os.environ["IFA_FUSE_ROWS"])))
         g = {"prefill_tok_s": {}, "params": int(sum(int(np.prod(s)) for s in synth.gelarax_tensor_shapes(cfg).values()))}
         for n in lens:
             prompt = [int(t) for t in rng.integers(3, 32000, n)]

@@ -463,6 +463,12 @@ int ifa_model_time_kernel(ifa_model *m, int which, int iters, float *avg_us);
 int ifa_linear_bf16w(const void *w_bf16, size_t rows, size_t cols, const void *a_f32, size_t lda, size_t tokens, const void *bias_bf16,
                      const void *mul_bf16, float alpha, int accumulate, int ops32, void *c_f32, size_t ldc, int silu_col0, int silu_col1,
                      ifa_stream stream);
+/* the same product for at most 8 rows (always the weight-streaming fp32 kernel) with the neighbouring element-wise op folded into the
+ * read of the activations: prologue 1 = layer norm without bias, a = (x - mean) / sqrt(var + eps) * norm_w[k]; prologue 2 = gated GELU,
+ * the row holds gate | up (lda >= 2 cols), a = gelu_tanh(gate[k]) * up[k]; 0 = none.  Needs cols % 8 == 0 and 16-byte aligned rows. */
+int ifa_linear_bf16w_rows(int prologue, const void *norm_w_bf16, float norm_eps, const void *w_bf16, size_t rows, size_t cols, const void *a_f32,
+                          size_t lda, size_t tokens, const void *bias_bf16, const void *mul_bf16, float alpha, int accumulate, void *c_f32,
+                          size_t ldc, int silu_col0, int silu_col1, ifa_stream stream);
 /* x[t] = embed[token_t] + pe(pos_t), pe[2i] = sin(p base^(-2i/width)), pe[2i+1] = cos(same); angles formed in double */
 int ifa_embed_sinpos_f32(const void *embed_bf16, int vocab, int width, const int *tokens_dev, const int *positions_dev, size_t tokens,
                          float base, void *x_f32, ifa_stream stream);

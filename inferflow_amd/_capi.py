@@ -149,6 +149,7 @@ SIGNATURES = {
     "ifa_model_tp_decode_batch": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _vp]),
     "ifa_model_get_tensor": (_i, [_vp, _i, _i, _vp, C.POINTER(_vp), C.POINTER(_sz), C.POINTER(_sz)]),
     "ifa_linear_bf16w": (_i, [_vp, _sz, _sz, _vp, _sz, _sz, _vp, _vp, _f, _i, _i, _vp, _sz, _i, _i, _vp]),
+    "ifa_linear_bf16w_rows": (_i, [_i, _vp, _f, _vp, _sz, _sz, _vp, _sz, _sz, _vp, _vp, _f, _i, _vp, _sz, _i, _i, _vp]),
     "ifa_embed_sinpos_f32": (_i, [_vp, _i, _i, _vp, _vp, _sz, _f, _vp, _vp]),
     "ifa_layernorm_f32": (_i, [_i, _vp, _sz, _sz, _sz, _vp, _f, _vp, _sz, _vp]),
     "ifa_glu_f32": (_i, [_i, _vp, _sz, _sz, _sz, _vp, _sz, _vp]),

@@ -10,6 +10,7 @@
 //             OPS32 = false: operands rounded to bfloat16, v_mfma_f32_32x32x16_bf16;
 //             OPS32 = true : operands stay 32-bit, v_mfma_f32_32x32x2_f32 (the exact mode of the worker)
 // Accumulation is fp32 in every path.  No atomics, no split K: a result does not depend on what else runs.
+#include <algorithm>
 #include "ifa_host.h"
 #include "ifa_f32_common.h"
 
@@ -27,6 +28,7 @@ struct LinArgs {
     int T, N, K, lda, ldc;
     float alpha; int accumulate, vec;
     int act_c0, act_c1;          // output columns [act_c0, act_c1) pass SiLU after the bias (projections whose consumer wants them activated)
+    const bf16_t *norm_w; float norm_eps;      // row kernel, prologue 1: the activations are layer-normed (no bias) on the fly
 };
 
 __device__ __forceinline__ void lin_store(const LinArgs &P, int t, int n, float acc)
@@ -129,12 +131,32 @@ __global__ void __launch_bounds__(256) k_lin_mfma(LinArgs P)
     }
 }
 
-// T <= TT rows; one wave per output row at a time
-template <int TT>
+// T <= TT rows; one wave per output row at a time.  PRO: what the activations pass as they are read (steps of a few rows are bound
+// by launches and dependent loads, not arithmetic, so the neighbouring element-wise launch is folded in here):
+//   1  layer norm without bias: a = (x - mean) / sqrt(var + eps) * w[k]   (every wave forms mean and variance of the T rows itself)
+//   2  gated GELU: the row holds gate | up (2 K values), a = gelu_tanh(gate[k]) * up[k]
+template <int TT, int PRO>
 __global__ void __launch_bounds__(256) k_lin_rows(LinArgs P)
 {
     const int lane = threadIdx.x & 63;
     const int wave = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6), nwaves = gridDim.x * (blockDim.x >> 6);
+    float mean[TT], rstd[TT];
+    if (PRO == 1) {
+#pragma unroll
+        for (int t = 0; t < TT; t++) {
+            const float *a = P.A + (size_t)min(t, P.T - 1) * P.lda;
+            float s = 0.0f;
+            for (int k = lane * 4; k < P.K; k += 256) { const float4 v = *reinterpret_cast<const float4 *>(a + k); s += (v.x + v.y) + (v.z + v.w); }
+            mean[t] = wave_sum(s) / (float)P.K;
+            float q = 0.0f;
+            for (int k = lane * 4; k < P.K; k += 256) {
+                const float4 v = *reinterpret_cast<const float4 *>(a + k);
+                const float d0 = v.x - mean[t], d1 = v.y - mean[t], d2 = v.z - mean[t], d3 = v.w - mean[t];
+                q += (d0 * d0 + d1 * d1) + (d2 * d2 + d3 * d3);
+            }
+            rstd[t] = 1.0f / sqrtf(wave_sum(q) / (float)P.K + P.norm_eps);
+        }
+    }
     for (int n = wave; n < P.N; n += nwaves) {
         float acc[TT];
 #pragma unroll
@@ -143,16 +165,31 @@ __global__ void __launch_bounds__(256) k_lin_rows(LinArgs P)
         if (P.vec) {
             for (int k = lane * 8; k < P.K; k += 512) {
                 const u32x4v wv = *reinterpret_cast<const u32x4v *>(w + k);
-                float w8[8];
+                float w8[8], g8[8];
 #pragma unroll
                 for (int e = 0; e < 4; e++) { w8[2 * e] = __uint_as_float(wv[e] << 16); w8[2 * e + 1] = __uint_as_float(wv[e] & 0xFFFF0000u); }
+                if (PRO == 1) {
+                    const u32x4v gv = *reinterpret_cast<const u32x4v *>(P.norm_w + k);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) { g8[2 * e] = __uint_as_float(gv[e] << 16); g8[2 * e + 1] = __uint_as_float(gv[e] & 0xFFFF0000u); }
+                }
 #pragma unroll
                 for (int t = 0; t < TT; t++) {
                     const float *a = P.A + (size_t)min(t, P.T - 1) * P.lda + k;
                     const float4 v0 = *reinterpret_cast<const float4 *>(a), v1 = *reinterpret_cast<const float4 *>(a + 4);
+                    float x8[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
+                    if (PRO == 1) {
+#pragma unroll
+                        for (int e = 0; e < 8; e++) x8[e] = (x8[e] - mean[t]) * rstd[t] * g8[e];
+                    } else if (PRO == 2) {
+                        const float4 u0 = *reinterpret_cast<const float4 *>(a + P.K), u1 = *reinterpret_cast<const float4 *>(a + P.K + 4);
+                        const float u8[8] = {u0.x, u0.y, u0.z, u0.w, u1.x, u1.y, u1.z, u1.w};
+#pragma unroll
+                        for (int e = 0; e < 8; e++) x8[e] = gelu_tanh_f(x8[e]) * u8[e];
+                    }
                     float s = acc[t];
-                    s = fmaf(v0.x, w8[0], s); s = fmaf(v0.y, w8[1], s); s = fmaf(v0.z, w8[2], s); s = fmaf(v0.w, w8[3], s);
-                    s = fmaf(v1.x, w8[4], s); s = fmaf(v1.y, w8[5], s); s = fmaf(v1.z, w8[6], s); s = fmaf(v1.w, w8[7], s);
+#pragma unroll
+                    for (int e = 0; e < 8; e++) s = fmaf(x8[e], w8[e], s);
                     acc[t] = s;
                 }
             }
@@ -173,27 +210,34 @@ __global__ void __launch_bounds__(256) k_lin_rows(LinArgs P)
 
 } // namespace
 
-extern "C" int ifa_linear_bf16w(const void *w_bf16, size_t rows, size_t cols, const void *a_f32, size_t lda, size_t tokens,
-                                const void *bias_bf16, const void *mul_bf16, float alpha, int accumulate, int ops32,
-                                void *c_f32, size_t ldc, int silu_col0, int silu_col1, ifa_stream stream)
+static int linear_launch(const void *w_bf16, size_t rows, size_t cols, const void *a_f32, size_t lda, size_t tokens, const void *bias_bf16,
+                         const void *mul_bf16, float alpha, int accumulate, int ops32, void *c_f32, size_t ldc, int silu_col0, int silu_col1, int prologue,
+                         const void *norm_w_bf16, float norm_eps, ifa_stream stream, const char *who)
 {
-    IFA_REQUIRE(w_bf16 && a_f32 && c_f32, "ifa_linear_bf16w: null pointer");
-    IFA_REQUIRE(rows > 0 && cols > 0 && tokens > 0 && lda >= cols && ldc >= rows, "ifa_linear_bf16w: bad shape (%zu x %zu, %zu tokens, lda %zu, ldc %zu)", rows, cols, tokens, lda, ldc);
-    IFA_REQUIRE(rows < (1u << 30) && cols < (1u << 30) && tokens < (1u << 30), "ifa_linear_bf16w: dimension too large");
+    IFA_REQUIRE(w_bf16 && a_f32 && c_f32, "%s: null pointer", who);
+    IFA_REQUIRE(rows > 0 && cols > 0 && tokens > 0 && lda >= cols * (prologue == 2 ? 2 : 1) && ldc >= rows, "%s: bad shape (%zu x %zu, %zu tokens, lda %zu, ldc %zu)", who, rows, cols, tokens, lda, ldc);
+    IFA_REQUIRE(rows < (1u << 30) && cols < (1u << 30) && tokens < (1u << 30), "%s: dimension too large", who);
     LinArgs P;
     P.W = (const bf16_t *)w_bf16; P.A = (const float *)a_f32; P.C = (float *)c_f32;
     P.bias = (const bf16_t *)bias_bf16; P.mul = (const bf16_t *)mul_bf16;
     P.T = (int)tokens; P.N = (int)rows; P.K = (int)cols; P.lda = (int)lda; P.ldc = (int)ldc;
     P.alpha = alpha; P.accumulate = accumulate ? 1 : 0; P.act_c0 = silu_col0; P.act_c1 = silu_col1;
+    P.norm_w = (const bf16_t *)norm_w_bf16; P.norm_eps = norm_eps;
     // 16-byte requests need whole 8-element pieces in every row of both operands
     P.vec = (cols % 8 == 0 && lda % 4 == 0 && ((uintptr_t)a_f32 & 15) == 0 && ((uintptr_t)w_bf16 & 15) == 0) ? 1 : 0;
     hipStream_t s = ifa_s(stream);
+    if (prologue) {
+        IFA_REQUIRE(prologue == 1 || prologue == 2, "%s: prologue %d", who, prologue);
+        IFA_REQUIRE(tokens <= 8 && P.vec, "%s: a fused prologue needs at most 8 rows and 16-byte aligned rows of whole 8-element pieces", who);
+        IFA_REQUIRE(prologue != 1 || (norm_w_bf16 && ((uintptr_t)norm_w_bf16 & 15) == 0), "%s: the norm's weight is missing or unaligned", who);
+    }
     if (tokens <= 8) {
         const unsigned grid = (unsigned)std::min<size_t>((rows + 3) / 4, 8192);
-        if (tokens == 1) hipLaunchKernelGGL(k_lin_rows<1>, dim3(grid), dim3(256), 0, s, P);
-        else if (tokens == 2) hipLaunchKernelGGL(k_lin_rows<2>, dim3(grid), dim3(256), 0, s, P);
-        else if (tokens <= 4) hipLaunchKernelGGL(k_lin_rows<4>, dim3(grid), dim3(256), 0, s, P);
-        else hipLaunchKernelGGL(k_lin_rows<8>, dim3(grid), dim3(256), 0, s, P);
+#define IFA_LR(TT) { if (prologue == 1) hipLaunchKernelGGL((k_lin_rows<TT, 1>), dim3(grid), dim3(256), 0, s, P); \
+                     else if (prologue == 2) hipLaunchKernelGGL((k_lin_rows<TT, 2>), dim3(grid), dim3(256), 0, s, P); \
+                     else hipLaunchKernelGGL((k_lin_rows<TT, 0>), dim3(grid), dim3(256), 0, s, P); }
+        if (tokens == 1) IFA_LR(1) else if (tokens == 2) IFA_LR(2) else if (tokens <= 4) IFA_LR(4) else IFA_LR(8)
+#undef IFA_LR
     } else {
         const dim3 grid(ifa_cdiv(rows, LM_N), ifa_cdiv(tokens, LM_T));
         if (ops32) hipLaunchKernelGGL(k_lin_mfma<true>, grid, dim3(256), 0, s, P);
@@ -201,4 +245,21 @@ extern "C" int ifa_linear_bf16w(const void *w_bf16, size_t rows, size_t cols, co
     }
     IFA_LAUNCH_CHECK();
     return IFA_OK;
+}
+
+extern "C" int ifa_linear_bf16w(const void *w_bf16, size_t rows, size_t cols, const void *a_f32, size_t lda, size_t tokens,
+                                const void *bias_bf16, const void *mul_bf16, float alpha, int accumulate, int ops32,
+                                void *c_f32, size_t ldc, int silu_col0, int silu_col1, ifa_stream stream)
+{
+    return linear_launch(w_bf16, rows, cols, a_f32, lda, tokens, bias_bf16, mul_bf16, alpha, accumulate, ops32, c_f32, ldc, silu_col0, silu_col1, 0, nullptr, 0.0f,
+                         stream, "ifa_linear_bf16w");
+}
+
+extern "C" int ifa_linear_bf16w_rows(int prologue, const void *norm_w_bf16, float norm_eps, const void *w_bf16, size_t rows, size_t cols, const void *a_f32,
+                                     size_t lda, size_t tokens, const void *bias_bf16, const void *mul_bf16, float alpha, int accumulate, void *c_f32,
+                                     size_t ldc, int silu_col0, int silu_col1, ifa_stream stream)
+{
+    IFA_REQUIRE(tokens <= 8, "ifa_linear_bf16w_rows: %zu rows (at most 8)", tokens);
+    return linear_launch(w_bf16, rows, cols, a_f32, lda, tokens, bias_bf16, mul_bf16, alpha, accumulate, 1, c_f32, ldc, silu_col0, silu_col1, prologue,
+                         norm_w_bf16, norm_eps, stream, "ifa_linear_bf16w_rows");
 }

@@ -57,10 +57,10 @@ __global__ void __launch_bounds__(256) k_glu_f32(int kind, const float *__restri
     out[(size_t)blockIdx.y * ldo + c] = act * u;
 }
 
-__global__ void __launch_bounds__(256) k_argmax_f32(const float *__restrict__ logits, int n, size_t row_stride, const int *__restrict__ excluded,
+__global__ void __launch_bounds__(1024) k_argmax_f32(const float *__restrict__ logits, int n, size_t row_stride, const int *__restrict__ excluded,
                                                     int *__restrict__ out)
 {
-    __shared__ float bv[4]; __shared__ int bi[4];
+    __shared__ float bv[16]; __shared__ int bi[16];
     const float *r = logits + (size_t)blockIdx.x * row_stride;
     int ex[3] = {-1, -1, -1};
     if (excluded) { const int ne = min(excluded[0], 3); for (int e = 0; e < ne; e++) ex[e] = excluded[1 + e]; }
@@ -77,7 +77,7 @@ __global__ void __launch_bounds__(256) k_argmax_f32(const float *__restrict__ lo
     if ((threadIdx.x & 63) == 0) { bv[threadIdx.x >> 6] = best; bi[threadIdx.x >> 6] = idx; }
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int w = 1; w < 4; w++) if (bv[w] > best || (bv[w] == best && bi[w] < idx)) { best = bv[w]; idx = bi[w]; }
+        for (int w = 1; w < (int)(blockDim.x >> 6); w++) if (bv[w] > best || (bv[w] == best && bi[w] < idx)) { best = bv[w]; idx = bi[w]; }
         out[blockIdx.x] = idx == 0x7FFFFFFF ? 0 : idx;
     }
 }
@@ -127,7 +127,7 @@ int ifa_glu_f32(int kind, const void *gate_up_f32, size_t ld, size_t rows, size_
 int ifa_argmax_rows_f32(const void *logits_f32, size_t n, size_t row_stride, size_t rows, const int *excluded_dev, int *out_dev, ifa_stream stream)
 {
     IFA_REQUIRE(logits_f32 && out_dev && n > 0 && rows > 0 && n < (1u << 30), "ifa_argmax_rows_f32: bad arguments");
-    hipLaunchKernelGGL(k_argmax_f32, dim3((unsigned)rows), dim3(256), 0, ifa_s(stream), (const float *)logits_f32, (int)n, row_stride, excluded_dev, out_dev);
+    hipLaunchKernelGGL(k_argmax_f32, dim3((unsigned)rows), dim3(n >= 4096 ? 1024 : 256), 0, ifa_s(stream), (const float *)logits_f32, (int)n, row_stride, excluded_dev, out_dev);
     IFA_LAUNCH_CHECK();
     return IFA_OK;
 }

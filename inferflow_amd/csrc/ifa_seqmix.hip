@@ -9,6 +9,7 @@
 // Everything that enters a recurrence is fp32; states live in fp32 in the slot arena of the worker (a table of one
 // base pointer per slot + an offset per layer).  A sequence that starts at position 0 starts from a zero state,
 // whatever the slot held before.
+#include <algorithm>
 #include "ifa_host.h"
 #include "ifa_f32_common.h"
 
@@ -16,21 +17,22 @@ using namespace ifa32;
 
 namespace {
 
-// grid: one workgroup per row.  y[t][c] = silu(sum_j w[c][j] in(i - (taps - 1) + j)[c]); in(idx) for idx < 0 comes from the
+// grid: (rows, channel slices).  y[t][c] = silu(sum_j w[c][j] in(i - (taps - 1) + j)[c]); in(idx) for idx < 0 comes from the
 // sequence's carried tail (rows [taps - 1][C], oldest first) or is zero at the start of a sequence.  Then channels
 // [0, norm_cols) are turned into unit vectors in groups of gdim (x / sqrt(sum x^2 + l2_eps)) and channels [0, scale_cols)
 // are multiplied by qscale.
 __global__ void __launch_bounds__(256) k_shortconv_silu(const float *__restrict__ x, size_t ldx, int C, int taps, const bf16_t *__restrict__ w,
                                                         const SeqDesc *__restrict__ seqs, const int *__restrict__ row_seq,
                                                         float *const *__restrict__ slot_base, size_t state_off, int norm_cols, int gdim,
-                                                        float l2_eps, int scale_cols, float qscale, float *__restrict__ y, size_t ldy)
+                                                        float l2_eps, int scale_cols, float qscale, float *__restrict__ y, size_t ldy, int slice)
 {
     extern __shared__ float ys[];
     const int t = blockIdx.x;
+    const int c_lo = blockIdx.y * slice, c_hi = min(C, c_lo + slice);      // this workgroup's channels (whole norm groups: slice % gdim == 0)
     const SeqDesc sd = seqs[row_seq[t]];
     const int i = t - sd.row0;
     const float *tail = sd.pos0 > 0 ? slot_base[sd.slot] + state_off : nullptr;
-    for (int c = threadIdx.x; c < C; c += blockDim.x) {
+    for (int c = c_lo + threadIdx.x; c < c_hi; c += blockDim.x) {
         float acc = 0.0f;
         for (int j = 0; j < taps; j++) {
             const int idx = i - (taps - 1) + j;
@@ -39,20 +41,20 @@ __global__ void __launch_bounds__(256) k_shortconv_silu(const float *__restrict_
             else v = tail ? tail[(size_t)(taps - 1 + idx) * C + c] : 0.0f;
             acc = fmaf(bf2f(w[(size_t)c * taps + j]), v, acc);
         }
-        ys[c] = silu_exact(acc);
+        ys[c - c_lo] = silu_exact(acc);
     }
     __syncthreads();
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
-    const int ngroups = gdim > 0 ? norm_cols / gdim : 0;
-    for (int gidx = wave; gidx < ngroups; gidx += nw) {
+    const int g_lo = gdim > 0 ? c_lo / gdim : 0, g_hi = gdim > 0 ? min(norm_cols, c_hi) / gdim : 0;
+    for (int gidx = g_lo + wave; gidx < g_hi; gidx += nw) {
         float s = 0.0f;
-        for (int e = lane; e < gdim; e += 64) { const float v = ys[gidx * gdim + e]; s = fmaf(v, v, s); }
+        for (int e = lane; e < gdim; e += 64) { const float v = ys[gidx * gdim + e - c_lo]; s = fmaf(v, v, s); }
         s = wave_sum(s);
         const float r = 1.0f / sqrtf(s + l2_eps);
-        for (int e = lane; e < gdim; e += 64) ys[gidx * gdim + e] *= r;
+        for (int e = lane; e < gdim; e += 64) ys[gidx * gdim + e - c_lo] *= r;
     }
     __syncthreads();
-    for (int c = threadIdx.x; c < C; c += blockDim.x) y[(size_t)t * ldy + c] = c < scale_cols ? ys[c] * qscale : ys[c];
+    for (int c = c_lo + threadIdx.x; c < c_hi; c += blockDim.x) y[(size_t)t * ldy + c] = c < scale_cols ? ys[c - c_lo] * qscale : ys[c - c_lo];
 }
 
 // grid: one workgroup per sequence.  The carried tail becomes the last taps - 1 inputs of (old tail, this step's rows).
@@ -322,10 +324,14 @@ int ifa_shortconv_silu_f32(const void *x_f32, size_t ldx, int channels, int taps
     IFA_REQUIRE(channels > 0 && taps >= 1 && taps <= 64 && rows > 0 && ldx >= (size_t)channels && ldy >= (size_t)channels, "ifa_shortconv_silu_f32: bad shape");
     IFA_REQUIRE(norm_cols >= 0 && norm_cols <= channels && scale_cols >= 0 && scale_cols <= channels && (norm_cols == 0 || (group_dim > 0 && norm_cols % group_dim == 0)),
                 "ifa_shortconv_silu_f32: bad norm groups");
-    IFA_REQUIRE((size_t)channels * 4 <= 64 * 1024, "ifa_shortconv_silu_f32: %d channels do not fit the LDS row", channels);
-    hipLaunchKernelGGL(k_shortconv_silu, dim3((unsigned)rows), dim3(256), (size_t)channels * 4, ifa_s(stream), (const float *)x_f32, ldx, channels, taps,
-                       (const bf16_t *)w_bf16, (const SeqDesc *)seqs_dev, row_seq_dev, (float *const *)slot_base_dev, state_off, norm_cols, group_dim, l2_eps,
-                       scale_cols, scale, (float *)y_f32, ldy);
+    // a row's channels go to several workgroups in slices of whole norm groups (~512 channels: steps of a few rows would otherwise
+    // leave the convolution to one workgroup)
+    const int gd = norm_cols > 0 ? group_dim : 1;
+    const int slice = std::min(channels, gd * std::max(1, (512 + gd - 1) / gd));
+    IFA_REQUIRE((size_t)slice * 4 <= 64 * 1024, "ifa_shortconv_silu_f32: norm groups of %d channels do not fit the LDS", group_dim);
+    hipLaunchKernelGGL(k_shortconv_silu, dim3((unsigned)rows, ifa_cdiv((size_t)channels, (size_t)slice)), dim3(256), (size_t)slice * 4, ifa_s(stream),
+                       (const float *)x_f32, ldx, channels, taps, (const bf16_t *)w_bf16, (const SeqDesc *)seqs_dev, row_seq_dev, (float *const *)slot_base_dev,
+                       state_off, norm_cols, group_dim, l2_eps, scale_cols, scale, (float *)y_f32, ldy, slice);
     IFA_LAUNCH_CHECK();
     return IFA_OK;
 }

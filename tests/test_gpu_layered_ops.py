@@ -105,17 +105,18 @@ def test_embedding_with_sinusoid_norms_glu_argmax():
     assert list(b) == [int(r.argmax()) for r in masked] and b[2] == 250
 
 
+@pytest.mark.parametrize("C_,gdim,nq,nsc", [(40, 8, 16, 8), (1100, 100, 600, 300)])      # (the second: a row's channels in two workgroups)
 @pytest.mark.parametrize("taps", [1, 2, 4])
-def test_short_convolution_with_carried_tail(taps):
+def test_short_convolution_with_carried_tail(taps, C_, gdim, nq, nsc):
     rng = np.random.default_rng(taps)
-    C_, gdim, nq = 40, 8, 16          # channels [0, 16) unit-normed in groups of 8, channels [0, 8) scaled
+    # channels [0, nq) unit-normed in groups of gdim, channels [0, nsc) scaled
     w = orc.bf16_round(0.5 * rng.standard_normal((C_, taps)))
     full = {s: rng.standard_normal((23, C_ + 5)).astype(np.float32) for s in (0, 1, 2)}
 
     def want(xs):
         y = orc.silu(orc.short_conv(orc.t64(xs[:, :C_]), orc.t64(w)))
         y[:, :nq] = orc.unit_vectors(y[:, :nq].reshape(-1, nq // gdim, gdim)).reshape(-1, nq)
-        y[:, :8] *= 0.25
+        y[:, :nsc] *= 0.25
         return y.numpy()
 
     sl = Slots(3, max(1, (taps - 1)) * C_)
@@ -128,7 +129,7 @@ def test_short_convolution_with_carried_tail(taps):
         d, rs, T = seq_tables(seqs)
         y = torch.empty((T, C_), dtype=torch.float32, device="cuda")
         xd = dev32(x)
-        ia.check(capi().ifa_shortconv_silu_f32(p(xd), C_ + 5, C_, taps, p(devbf(w)), p(d), p(rs), T, p(sl.table), 0, nq, gdim, 1e-6, 8, 0.25, p(y), C_, stream()))
+        ia.check(capi().ifa_shortconv_silu_f32(p(xd), C_ + 5, C_, taps, p(devbf(w)), p(d), p(rs), T, p(sl.table), 0, nq, gdim, 1e-6, nsc, 0.25, p(y), C_, stream()))
         ia.check(capi().ifa_shortconv_tail_f32(p(xd), C_ + 5, C_, taps, p(d), len(seqs), p(sl.table), 0, stream()))
         sync()
         got, r = y.cpu().numpy(), 0
@@ -139,7 +140,7 @@ def test_short_convolution_with_carried_tail(taps):
     new = rng.standard_normal((4, C_ + 5)).astype(np.float32)
     d, rs, T = seq_tables([(4, 0, 2)])
     y = torch.empty((T, C_), dtype=torch.float32, device="cuda")
-    ia.check(capi().ifa_shortconv_silu_f32(p(dev32(new)), C_ + 5, C_, taps, p(devbf(w)), p(d), p(rs), T, p(sl.table), 0, nq, gdim, 1e-6, 8, 0.25, p(y), C_, stream()))
+    ia.check(capi().ifa_shortconv_silu_f32(p(dev32(new)), C_ + 5, C_, taps, p(devbf(w)), p(d), p(rs), T, p(sl.table), 0, nq, gdim, 1e-6, nsc, 0.25, p(y), C_, stream()))
     assert np.abs(y.cpu().numpy() - want(new)).max() < 1e-5
 
 
@@ -276,3 +277,25 @@ def test_windowed_attention_tiles_over_several_sequences():
         for s_, n in step:
             assert np.abs(got[r:r + n] - want[s_][at[s_]:at[s_] + n]).max() < 2e-5 * max(1.0, np.abs(want[s_]).max()), (s_, at[s_], n)
             r += n; at[s_] += n
+
+
+@pytest.mark.parametrize("T", [1, 2, 3, 5, 8])
+def test_row_products_with_the_norm_or_the_gated_gelu_folded_in(T):
+    rng = np.random.default_rng(40 + T)
+    N, K = 77, 96
+    W = orc.bf16_round(rng.standard_normal((N, K)) / 8)
+    bias, mul, g = (orc.bf16_round(rng.standard_normal(n)) for n in (N, N, K))
+    x = (2 * rng.standard_normal((T, K + 4)) + 1).astype(np.float32)
+    c0 = rng.standard_normal((T, N)).astype(np.float32)
+    c = dev32(c0)
+    ia.check(capi().ifa_linear_bf16w_rows(1, p(devbf(g)), 1e-5, p(devbf(W)), N, K, p(dev32(x)), K + 4, T, p(devbf(bias)), p(devbf(mul)), 0.5, 1, p(c), N, 3, 9, stream()))
+    h = orc.layer_norm_nobias(orc.t64(x[:, :K]), orc.t64(g), 1e-5)
+    want = h @ orc.t64(W).T + orc.t64(bias)
+    want[:, 3:9] = orc.silu(want[:, 3:9])
+    want = (want * orc.t64(mul) * 0.5 + orc.t64(c0)).numpy()
+    assert np.abs(c.cpu().numpy() - want).max() < 2e-5 * max(1.0, np.abs(want).max())
+    gu = (2 * rng.standard_normal((T, 2 * K + 4))).astype(np.float32)
+    c = torch.empty((T, N), dtype=torch.float32, device="cuda")
+    ia.check(capi().ifa_linear_bf16w_rows(2, None, 0.0, p(devbf(W)), N, K, p(dev32(gu)), 2 * K + 4, T, None, None, 1.0, 0, p(c), N, 0, 0, stream()))
+    want = ((orc.gelu_tanh(orc.t64(gu[:, :K])) * orc.t64(gu[:, K:2 * K])) @ orc.t64(W).T).numpy()
+    assert np.abs(c.cpu().numpy() - want).max() < 2e-5 * max(1.0, np.abs(want).max())
