@@ -318,7 +318,8 @@ bool InferenceEngine::Init(const InferenceConfig &cfg)
     perf_phases_ = !multi_ && config_.debug.is_study_mode && config_.debug.enable_perf_stat;
     if (perf_phases_ && ifa_model_set_option(model_, "perf_stat", 1) != IFA_OK) { EngineSetError("perf_stat: %s", ifa_last_error()); Clear(); return false; }
     // one KV cache per concurrent query, like the reference's per-query LayerKVCache sets
-    kv_slots_ = std::max(1, std::min(config_.max_concurrent_queries, 64));
+    // (a layer-list worker allocates a slot's memory when the slot is first used: its limit is the table of slots, not memory up front)
+    kv_slots_ = std::max(1, std::min(config_.max_concurrent_queries, !multi_ && ifa_model_is_layered(model_) ? 4096 : 64));
     {
         std::vector<ifa_model *> all;
         if (multi_) for (WorkerPlan &w : multi_->plans) all.push_back(w.model); else all.push_back(model_);

@@ -23,7 +23,7 @@ using namespace inferflow_amd;
 int main(int argc, char **argv)
 {
     std::string model, dtype = "bfloat16", out;
-    int max_tokens = 4096, max_queries = 64;
+    int max_tokens = 4096, max_queries = 1024;
     for (int i = 1; i < argc; i++) {
         const std::string a = argv[i];
         auto next = [&]() -> const char * { return i + 1 < argc ? argv[++i] : ""; };

@@ -207,7 +207,7 @@ def test_delta_gates_and_gated_group_norm():
 
 
 @pytest.mark.parametrize("tile_min", [16, 1 << 30])       # prompts through the tiled matrix-core kernel / every row through the per-row kernel
-@pytest.mark.parametrize("heads,kv_heads,dim,window,keep,nb,dmax", [(4, 2, 16, 9, 2, 8, 30), (2, 2, 8, 1, 0, 4, 6), (3, 1, 68, 300, 5, 32, 240), (6, 3, 32, 17, 40, 10, 12),
+@pytest.mark.parametrize("heads,kv_heads,dim,window,keep,nb,dmax", [(4, 2, 16, 9, 2, 8, 30), (2, 2, 8, 1, 0, 4, 6), (3, 1, 68, 300, 5, 24, 200), (6, 3, 32, 17, 40, 10, 12),
                                                                     (2, 1, 64, 20, 3, 8, 30), (2, 1, 32, 2000, 4, 8, 30), (2, 2, 128, 50, 0, 16, 100), (1, 1, 96, 9, 2, 8, 30), (4, 2, 64, 33, 33, 6, 7)])
 def test_windowed_attention_with_sink_cap_and_bucket_bias(heads, kv_heads, dim, window, keep, nb, dmax, tile_min):
     rng = np.random.default_rng(heads + dim + window)

@@ -33,8 +33,8 @@ def test_layered_only_library_builds_and_declines_the_standard_network():
 
 def test_oracle_bucket_map_and_visibility():
     assert [orc.distance_bucket(n, 8, 32) for n in (0, 1, 3, 4, 5, 31, 32, 500)] == [0, 1, 3, 4, 4, 7, 7, 7]
-    rows = [orc.distance_bucket(n, 32, 240) for n in range(400)]
-    assert rows[:16] == list(range(16)) and all(b >= a for a, b in zip(rows, rows[1:])) and rows[240] == 31 and rows[239] == 31 and max(rows) == 31
+    rows = [orc.distance_bucket(n, 24, 100) for n in range(300)]
+    assert rows[:12] == list(range(12)) and all(b >= a for a, b in zip(rows, rows[1:])) and rows[100] == 23 and rows[99] == 23 and max(rows) == 23
     v = orc.visible(12, 4, 2).numpy()
     assert v[11].tolist() == [True, True] + [False] * 6 + [True] * 4 and v[3].tolist() == [True] * 4 + [False] * 8
 
