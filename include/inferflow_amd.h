@@ -517,7 +517,7 @@ int ifa_kv_store_f32(const void *k_f32, size_t ldk, const void *v_f32, size_t ld
  * Steps of at least tile_min_rows rows (head sizes 32 / 64 / 96 / 128) take the tiled kernel -- 128 queries of one sequence per workgroup,
  * scores and weighted sums on the fp32 matrix cores -- which needs the step's sequences on the host too (seqs_host [n_seqs], the same
  * values as seqs_dev; NULL / n_seqs 0: always one workgroup per row).  With a workspace (ws_f32, ws_bytes; nullable) and at most 512
- * (row, head) pairs, the keys of a pair are shared out to up to 16 workgroups and merged by a second launch (decode steps). */
+ * (row, head) pairs, the keys of a pair are shared out to up to 32 workgroups (64 keys each) and merged by a second launch (decode steps). */
 int ifa_attention_window_f32(const void *q_f32, size_t ldq, int heads, int kv_heads, int dim, int norm_q, float eps, float scale, float softcap,
                              int window, int keep_first, const void *rel_bf16, const int *bucket_of_dev, int n_buckets, const void *sink_bf16,
                              const void *seqs_dev, const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t k_off, size_t v_off,

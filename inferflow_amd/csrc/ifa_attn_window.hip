@@ -145,23 +145,29 @@ __global__ void __launch_bounds__(256) k_attn_window(WinAttnArgs P)
     }
 }
 
-// grid (rows, heads): the shares of a (row, head) and its sink into the output row
+// grid (rows, heads), one wave: the shares of a (row, head) and its sink into the output row.  Lane sp holds share sp's maximum and
+// sum, so the scale factors come from two wave reductions; the weighted values are then read for all shares at once.
+constexpr int WA_MAX_SPLITS = 32;
+
 __global__ void __launch_bounds__(64) k_attn_window_combine(WinAttnArgs P)
 {
-    const int t = blockIdx.x, h = blockIdx.y, dim = P.dim, nsplit = P.nsplit;
+    const int t = blockIdx.x, h = blockIdx.y, dim = P.dim, nsplit = P.nsplit, lane = threadIdx.x;
     const float *src = P.ws + ((size_t)t * P.heads + h) * nsplit * (dim + 2);
     const float snk = P.sink ? bf2f(P.sink[h]) : -INFINITY;
-    float M = snk;
-    for (int sp = 0; sp < nsplit; sp++) M = fmaxf(M, src[(size_t)sp * (dim + 2)]);
-    float L = P.sink ? expf(snk - M) : 0.0f;
-    for (int sp = 0; sp < nsplit; sp++) { const float m = src[(size_t)sp * (dim + 2)]; if (m != -INFINITY) L += src[(size_t)sp * (dim + 2) + 1] * expf(m - M); }
-    for (int d = threadIdx.x; d < dim; d += blockDim.x) {
+    const float m_sp = lane < nsplit ? src[(size_t)lane * (dim + 2)] : -INFINITY, l_sp = lane < nsplit ? src[(size_t)lane * (dim + 2) + 1] : 0.0f;
+    const float M = fmaxf(snk, wave_max(m_sp));
+    const float f_sp = m_sp == -INFINITY ? 0.0f : expf(m_sp - M);
+    const float L = wave_sum(l_sp * f_sp) + (P.sink ? expf(snk - M) : 0.0f);
+    for (int d = lane; d < dim; d += 64) {
+        float v[WA_MAX_SPLITS];
+#pragma unroll
+        for (int sp = 0; sp < WA_MAX_SPLITS; sp++) v[sp] = sp < nsplit ? src[(size_t)sp * (dim + 2) + 2 + d] : 0.0f;
         float o = 0.0f;
-        for (int sp = 0; sp < nsplit; sp++) { const float m = src[(size_t)sp * (dim + 2)]; if (m != -INFINITY) o = fmaf(src[(size_t)sp * (dim + 2) + 2 + d], expf(m - M), o); }
+#pragma unroll
+        for (int sp = 0; sp < WA_MAX_SPLITS; sp++) o = fmaf(v[sp], __shfl(f_sp, sp, 64), o);
         P.out[(size_t)t * P.ldo + (size_t)h * dim + d] = o / L;
     }
 }
-
 
 // ---- prompts: 128 queries of one sequence per workgroup, the visible keys walked in blocks of 32 that are staged ONCE per workgroup
 // in LDS; each wave owns 32 queries: S = Q K^T and O += P V on the fp32 matrix cores (v_mfma_f32_32x32x2_f32: scores and weights
@@ -349,7 +355,7 @@ int ifa_attention_window_f32(const void *q_f32, size_t ldq, int heads, int kv_he
     // few rows: a (row, head)'s keys are shared out to several workgroups (one workgroup pulls its keys through ONE compute unit)
     int nsplit = 1;
     if (ws_f32 && rows * (size_t)heads <= 512) {
-        nsplit = (int)std::min<size_t>(16, ((size_t)window + (size_t)keep_first + 127) / 128);
+        nsplit = (int)std::min<size_t>(WA_MAX_SPLITS, ((size_t)window + (size_t)keep_first + 63) / 64);
         while (nsplit > 1 && rows * (size_t)heads * nsplit * ((size_t)dim + 2) * 4 > ws_bytes) nsplit--;
     }
     P.ws = (float *)ws_f32; P.nsplit = nsplit;

@@ -402,7 +402,7 @@ int lay_finalize(ifa_model *m)
     if (!n->attn_ws) {
         size_t per_row = 0;
         for (const LLayer &L : n->layers)
-            if (L.spec.mixer == IFA_MIX_WINDOW_LINEAR) per_row = std::max(per_row, (size_t)L.spec.a_heads * 16 * ((size_t)L.spec.a_dim + 2) * 4);
+            if (L.spec.mixer == IFA_MIX_WINDOW_LINEAR) per_row = std::max(per_row, (size_t)L.spec.a_heads * 32 * ((size_t)L.spec.a_dim + 2) * 4);
         n->attn_ws_bytes = per_row * 64;
         if (n->attn_ws_bytes) IFA_HIP_CHECK(hipMalloc((void **)&n->attn_ws, n->attn_ws_bytes));
     }

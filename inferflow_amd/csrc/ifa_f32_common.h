@@ -47,6 +47,14 @@ __device__ __forceinline__ float quad_sum(float v)
     return v;
 }
 
+// sum over the eight lanes 8 q .. 8 q + 7: the quad sums, then the other quad's through a half-row mirror (lane i <-> 7 - i)
+__device__ __forceinline__ float oct_sum(float v)
+{
+    v = quad_sum(v);
+    v += __int_as_float(__builtin_amdgcn_mov_dpp(__float_as_int(v), 0x141, 0xF, 0xF, true));
+    return v;
+}
+
 // sum over a workgroup of up to 1024 threads; red: 17 floats of LDS; every thread gets the result
 __device__ __forceinline__ float block_sum(float v, float *red)
 {

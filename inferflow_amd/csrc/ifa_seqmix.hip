@@ -164,23 +164,23 @@ __global__ void __launch_bounds__(64) k_state_scan(ScanArgs P)
     if (live) for (int i = 0; i < dk; i++) state[(size_t)i * P.dv + j] = S[i * 64 + lane];
 }
 
-// The same recurrences for key sizes 32 / 64 / 128 with the state in REGISTERS and FOUR lanes per column: lane 4 c + r of a wave owns
-// rows [r DK / 4, (r + 1) DK / 4) of column c (16 columns per wave), so a token is DK / 4 elements of dependent arithmetic per lane
+// The same recurrences for key sizes 16 / 32 / 64 / 128 with the state in REGISTERS and FOUR (key sizes from 64 on: EIGHT) lanes per column:
+// lane 4 c + r of a wave owns rows [r DK / 4, (r + 1) DK / 4) of column c (16 columns per wave), so a token is DK / 4 elements of dependent arithmetic per lane
 // instead of DK -- the recurrence is a chain of dependent instructions of a wave that is alone on its SIMD, and its length per token
 // is what the prompt rate of these layers comes down to.  The sums over a column's rows (the read-out, and S^T k of the delta rule)
-// are finished across the four lanes by two DPP quad permutes.  Tokens go in groups of 8: the group's q, k and gates are staged in
+// are finished across the lanes of a column by two DPP quad permutes (+ one half-row mirror for eight lanes).  Tokens go in groups of 8: the group's q, k and gates are staged in
 // LDS (16-byte reads of a lane's row range), the next group's operands are requested from memory before the current group is
 // computed.  fp32 results differ from the general kernel's by the order of these sums only.
 constexpr int SCAN_TB = 8;
 
-template <int KIND, int DK>
+template <int KIND, int DK, int LPC>
 __global__ void __launch_bounds__(64) k_state_scan_reg(ScanArgs P)
 {
-    constexpr int DKQ = DK / 4;
+    constexpr int DKQ = DK / LPC, CPW = 64 / LPC;      // rows per lane, columns per wave
     __shared__ __attribute__((aligned(16))) float qs[2][SCAN_TB][DK], ks[2][SCAN_TB][DK];
     __shared__ float gs[2][SCAN_TB], bs[2][SCAN_TB];
     const int seq = blockIdx.x / P.heads, h = blockIdx.x % P.heads;
-    const int lane = threadIdx.x, rg = lane & 3, j = blockIdx.y * 16 + (lane >> 2);
+    const int lane = threadIdx.x, rg = lane & (LPC - 1), j = blockIdx.y * CPW + lane / LPC;
     const bool live = j < P.dv;
     const int jc = live ? j : P.dv - 1;
     const int qh = h / (P.heads / P.qk_heads);
@@ -255,14 +255,14 @@ __global__ void __launch_bounds__(64) k_state_scan_reg(ScanArgs P)
                         S[e] *= gt; r0 = fmaf(S[e], kk[e], r0);
                         S[e + 1] *= gt; r1 = fmaf(S[e + 1], kk[e + 1], r1);
                     }
-                    const float u = bt * (vt - quad_sum(r0 + r1));
+                    const float u = bt * (vt - (LPC == 8 ? oct_sum(r0 + r1) : quad_sum(r0 + r1)));
 #pragma unroll
                     for (int e = 0; e < DKQ; e += 2) {
                         S[e] = fmaf(kk[e], u, S[e]); o0 = fmaf(S[e], qq[e], o0);
                         S[e + 1] = fmaf(kk[e + 1], u, S[e + 1]); o1 = fmaf(S[e + 1], qq[e + 1], o1);
                     }
                 }
-                const float o = quad_sum(o0 + o1);
+                const float o = LPC == 8 ? oct_sum(o0 + o1) : quad_sum(o0 + o1);
                 if (live && rg == 0) P.out[(size_t)(sd.row0 + t0 + tt) * P.ldo + (size_t)h * P.dv + j] = o;
             }
         }
@@ -376,11 +376,15 @@ int ifa_state_scan_f32(int kind, int in_act, const void *q_f32, size_t ldq, cons
     P.out = (float *)out_f32; P.ldo = ldo;
     const size_t smem = ((size_t)dk * 64 + 2 * (size_t)dk) * 4;
     const dim3 grid((unsigned)(n_seqs * heads), ifa_cdiv((size_t)dv, 64));
-    const dim3 grid16((unsigned)(n_seqs * heads), ifa_cdiv((size_t)dv, 16));
+    // four lanes per column (16 columns per wave); key sizes from 64 on: eight lanes per column (8 columns per wave)
+    const dim3 grid16((unsigned)(n_seqs * heads), ifa_cdiv((size_t)dv, 16)), grid8((unsigned)(n_seqs * heads), ifa_cdiv((size_t)dv, 8));
 #define IFA_SCAN_REG(DKV) \
     if (dk == DKV) { \
-        if (kind == 0) hipLaunchKernelGGL((k_state_scan_reg<0, DKV>), grid16, dim3(64), 0, ifa_s(stream), P); \
-        else hipLaunchKernelGGL((k_state_scan_reg<1, DKV>), grid16, dim3(64), 0, ifa_s(stream), P); \
+        if (DKV >= 64) { \
+            if (kind == 0) hipLaunchKernelGGL((k_state_scan_reg<0, DKV, 8>), grid8, dim3(64), 0, ifa_s(stream), P); \
+            else hipLaunchKernelGGL((k_state_scan_reg<1, DKV, 8>), grid8, dim3(64), 0, ifa_s(stream), P); \
+        } else if (kind == 0) hipLaunchKernelGGL((k_state_scan_reg<0, DKV, 4>), grid16, dim3(64), 0, ifa_s(stream), P); \
+        else hipLaunchKernelGGL((k_state_scan_reg<1, DKV, 4>), grid16, dim3(64), 0, ifa_s(stream), P); \
         IFA_LAUNCH_CHECK(); \
         return IFA_OK; \
     }

@@ -208,7 +208,7 @@ def test_delta_gates_and_gated_group_norm():
 
 @pytest.mark.parametrize("tile_min", [16, 1 << 30])       # prompts through the tiled matrix-core kernel / every row through the per-row kernel
 @pytest.mark.parametrize("heads,kv_heads,dim,window,keep,nb,dmax", [(4, 2, 16, 9, 2, 8, 30), (2, 2, 8, 1, 0, 4, 6), (3, 1, 68, 300, 5, 24, 200), (6, 3, 32, 17, 40, 10, 12),
-                                                                    (2, 1, 64, 20, 3, 8, 30), (2, 1, 32, 2000, 4, 8, 30), (2, 2, 128, 50, 0, 16, 100), (1, 1, 96, 9, 2, 8, 30), (4, 2, 64, 33, 33, 6, 7)])
+                                                                    (2, 1, 64, 20, 3, 8, 30), (2, 1, 32, 2000, 4, 8, 30), (2, 2, 128, 50, 0, 16, 100), (1, 1, 96, 9, 2, 8, 30), (4, 2, 64, 33, 33, 6, 7), (8, 2, 16, 12, 1, 8, 30), (8, 1, 32, 25, 2, 8, 30)])
 def test_windowed_attention_with_sink_cap_and_bucket_bias(heads, kv_heads, dim, window, keep, nb, dmax, tile_min):
     rng = np.random.default_rng(heads + dim + window)
     L, eps, scale, cap = 150, 1e-6, 0.3, 6.0
@@ -225,7 +225,7 @@ def test_windowed_attention_with_sink_cap_and_bucket_bias(heads, kv_heads, dim, 
     bucket_of = devi([orc.distance_bucket(n, nb, dmax) for n in range(ctx)])
     kvd = kv_heads * dim
     sl = Slots(2, 2 * ctx * kvd)
-    ws = torch.full((2 * heads * 16 * (dim + 2),), float('nan'), dtype=torch.float32, device='cuda')      # single tokens: the keys shared out over workgroups
+    ws = torch.full((2 * heads * 32 * (dim + 2),), float('nan'), dtype=torch.float32, device='cuda')      # single tokens: the keys shared out over workgroups
     at = 0
     for n in (1, 2, 60, 1, 1, 80, 5):                # prompt portions and single tokens; the same sequence lives on slot 1
         d, rs, T = seq_tables([(n, at, 1)])
