@@ -197,7 +197,7 @@ def test_far_key_among_hundreds_and_long_decoding(tmp_path):
     eng.close()
 
 
-@pytest.mark.parametrize("case", ["gqa_1", "mha", "delta_first_taps2", "no_ffn_anywhere", "odd_sizes"])
+@pytest.mark.parametrize("case", ["gqa_1", "mha", "delta_first_taps2", "no_ffn_anywhere", "odd_sizes", "tiny_unaligned", "wide_heads"])
 def test_other_sizes(tmp_path, case):
     if case == "gqa_1":
         cfg = fx.config([fx.parallel_layer(heads=4, kv_heads=1, dim=8, window=1, keep_first=1, lin_heads=1, lin_dim=4, lin_vdim=4, ff=16)], width=16, vocab=11)
@@ -209,6 +209,14 @@ def test_other_sizes(tmp_path, case):
                          fx.parallel_layer()], width=40, vocab=29)
     elif case == "no_ffn_anywhere":
         cfg = fx.config([fx.parallel_layer(ff=0), fx.delta_layer(ff=0)], width=24, vocab=19)
+    elif case == "tiny_unaligned":
+        cfg = fx.config([fx.parallel_layer(heads=2, kv_heads=1, dim=6, window=5, keep_first=1, lin_heads=1, lin_dim=3, lin_vdim=5, ff=10),
+                         fx.delta_layer(heads=2, kv_heads=2, dim=6, vdim=5, conv=3, ff=0)], width=14, vocab=9)
+    elif case == "wide_heads":
+        cfg = fx.config([fx.parallel_layer(heads=2, kv_heads=1, dim=160, window=30, keep_first=2, lin_heads=1, lin_dim=128, lin_vdim=96, ff=64),
+                         fx.delta_layer(heads=2, kv_heads=1, dim=64, vdim=72, conv=4, ff=64), fx.parallel_layer(heads=4, kv_heads=4, dim=32, window=7, keep_first=9,
+                                                                                                              lin_heads=2, lin_dim=32, lin_vdim=16, ff=0)],
+                        width=128, vocab=50)
     else:
         cfg = fx.config([fx.parallel_layer(heads=5, kv_heads=5, dim=20, window=13, keep_first=2, lin_heads=3, lin_dim=12, lin_vdim=36, ff=52),
                          fx.delta_layer(heads=5, kv_heads=1, dim=12, vdim=20, conv=4, ff=52)], width=36, vocab=23)
