@@ -4,6 +4,8 @@ describe the same thing."""
 import ctypes as C
 import os
 import shutil
+import subprocess
+import sys
 
 import numpy as np
 import pytest
@@ -19,15 +21,22 @@ def test_layered_only_library_builds_and_declines_the_standard_network():
     from inferflow_amd import build
     path = build.build_layered_library()
     assert os.path.exists(path) and os.path.exists(build.LAYERED_CLI_PATH)
-    L = C.CDLL(path)
-    for name in ("ifa_model_create_layered", "ifa_model_set_tensor_host", "ifa_model_step_seqs", "ifa_model_logits_f32", "ifa_model_forward",
-                 "ifa_model_decode", "ifa_model_decode_batch", "ifa_model_kv_slots", "ifa_model_select_kv", "ifa_model_finalize", "ifa_model_destroy",
-                 "ifa_engine_create_from_dir", "ifa_engine_infer", "ifa_engine_commit", "ifa_engine_last_logits_f32", "ifa_linear_bf16w",
-                 "ifa_attention_window_f32", "ifa_state_scan_f32", "ifa_shortconv_silu_f32"):
-        assert hasattr(L, name), name
-    L.ifa_last_error.restype = C.c_char_p
-    out = C.c_void_p()
-    assert L.ifa_model_create(None, C.byref(out)) != 0 and b"standard network" in L.ifa_last_error()
+    # in a process of its own: another test may have loaded the full library with RTLD_GLOBAL, and its symbols would answer first
+    code = ("import ctypes as C, sys\n"
+            "L = C.CDLL(sys.argv[1])\n"
+            "names = sys.argv[2].split(',')\n"
+            "missing = [n for n in names if not hasattr(L, n)]\n"
+            "L.ifa_last_error.restype = C.c_char_p\n"
+            "out = C.c_void_p()\n"
+            "rc = L.ifa_model_create(None, C.byref(out))\n"
+            "print(missing, rc, L.ifa_last_error().decode())\n")
+    names = ("ifa_model_create_layered", "ifa_model_set_tensor_host", "ifa_model_step_seqs", "ifa_model_logits_f32", "ifa_model_forward",
+             "ifa_model_decode", "ifa_model_decode_batch", "ifa_model_kv_slots", "ifa_model_select_kv", "ifa_model_finalize", "ifa_model_destroy",
+             "ifa_engine_create_from_dir", "ifa_engine_infer", "ifa_engine_commit", "ifa_engine_last_logits_f32", "ifa_linear_bf16w",
+             "ifa_attention_window_f32", "ifa_state_scan_f32", "ifa_shortconv_silu_f32")
+    r = subprocess.run([sys.executable, "-c", code, path, ",".join(names)], capture_output=True, text=True, timeout=120)
+    assert r.returncode == 0, r.stderr[-2000:]
+    assert r.stdout.startswith("[] -4 ") and "standard network" in r.stdout, r.stdout
     assert os.access(os.path.join(ROOT, "bin", "trace_run"), os.X_OK)
 
 
