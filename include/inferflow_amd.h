@@ -250,6 +250,7 @@ typedef struct {
 /* tensor ids for ifa_model_set_tensor (StdDeviceNetwork, src/transformer/model.h:168-276) */
 enum {
     IFA_T_EMBD = 0, IFA_T_OUT_NORM = 1, IFA_T_OUT_NORM_B = 2, IFA_T_LM_HEAD = 3,
+    IFA_T_EMBD_NORM = 4,      /* layer-list models with stem 1: weight of the grouped RMS norm behind the embedding */
     IFA_T_ATTN_NORM = 10, IFA_T_ATTN_NORM_B = 11, IFA_T_WQ = 12, IFA_T_WK = 13, IFA_T_WV = 14, IFA_T_WO = 15,
     IFA_T_FFN_NORM = 16, IFA_T_FFN_NORM_B = 17, IFA_T_W1 = 18, IFA_T_W2 = 19, IFA_T_W3 = 20, IFA_T_MOE_GATE = 21,
     IFA_T_WQ_B = 22, IFA_T_WK_B = 23, IFA_T_WV_B = 24, IFA_T_WO_B = 25, IFA_T_W1_B = 26, IFA_T_W2_B = 27, IFA_T_W3_B = 28,
@@ -469,6 +470,12 @@ int ifa_linear_bf16w(const void *w_bf16, size_t rows, size_t cols, const void *a
 int ifa_linear_bf16w_rows(int prologue, const void *norm_w_bf16, float norm_eps, const void *w_bf16, size_t rows, size_t cols, const void *a_f32,
                           size_t lda, size_t tokens, const void *bias_bf16, const void *mul_bf16, float alpha, int accumulate, void *c_f32,
                           size_t ldc, int silu_col0, int silu_col1, ifa_stream stream);
+/* Grouped product on the matrix cores: `groups` matrices [rows][cols] back to back in w_bf16; the output rows are sorted by group and cut
+ * into tiles of at most 64 rows of ONE group: tile_map_dev[3 i] = {group, first row, rows}, *n_tiles_dev tiles (max_tiles < 65536 bounds
+ * the grid).  C[r][n] = row_scale[r] * act(sum_k A[a_rows[r]][k] W_group[n][k]); a_rows_dev / row_scale_f32 nullable; act 0 none, 1 erf-GELU. */
+int ifa_linear_bf16w_grouped(const void *w_bf16, size_t rows, size_t cols, int groups, const void *a_f32, size_t lda, const int *a_rows_dev,
+                             const int *tile_map_dev, const int *n_tiles_dev, size_t max_tiles, const void *row_scale_f32, int act, int ops32,
+                             void *c_f32, size_t ldc, ifa_stream stream);
 /* x[t] = embed[token_t] + pe(pos_t), pe[2i] = sin(p base^(-2i/width)), pe[2i+1] = cos(same); angles formed in double */
 int ifa_embed_sinpos_f32(const void *embed_bf16, int vocab, int width, const int *tokens_dev, const int *positions_dev, size_t tokens,
                          float base, void *x_f32, ifa_stream stream);
@@ -513,7 +520,7 @@ int ifa_kv_store_f32(const void *k_f32, size_t ldk, const void *v_f32, size_t ld
 /* softmax attention of the step's rows over their sequences' caches: query i sees key j iff j <= i and (i - j < window or
  * j < keep_first); q RMS-normed per head if norm_q; score = q.k * scale, soft cap cap * tanh(score / cap) if softcap > 0, + bias
  * rel[bucket_of[i - j]][head] if rel (bf16 [n_buckets][heads], bucket_of_dev: int per distance 0 .. max_ctx - 1); sink_bf16 [heads]
- * (nullable): exp(sink) joins the denominator.  dim <= 256.  out fp32 [rows][heads * dim].
+ * (nullable): exp(sink) joins the denominator.  dim <= 640.  out fp32 [rows][heads * dim].
  * Steps of at least tile_min_rows rows (head sizes 32 / 64 / 96 / 128) take the tiled kernel -- 128 queries of one sequence per workgroup,
  * scores and weighted sums on the fp32 matrix cores -- which needs the step's sequences on the host too (seqs_host [n_seqs], the same
  * values as seqs_dev; NULL / n_seqs 0: always one workgroup per row).  With a workspace (ws_f32, ws_bytes; nullable) and at most 512
@@ -523,6 +530,61 @@ int ifa_attention_window_f32(const void *q_f32, size_t ldq, int heads, int kv_he
                              const void *seqs_dev, const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t k_off, size_t v_off,
                              void *out_f32, size_t ldo, const void *seqs_host, int n_seqs, int tile_min_rows, void *ws_f32, size_t ws_bytes, ifa_stream stream);
 
+/* x[t] = embed[token_t] (bf16 rows) as fp32, no position vector */
+int ifa_embed_rows_f32(const void *embed_bf16, int vocab, int width, const int *tokens_dev, size_t tokens, void *x_f32, ifa_stream stream);
+/* RMS norm in `groups` equal consecutive parts of a row: y = x / sqrt(mean_part(x^2) + eps) * w[c]; accumulate != 0: y += that (the
+ * residual update of a block whose norm sits on the sub-layer's OUTPUT).  cols % groups == 0; y may be x when accumulate == 0. */
+int ifa_group_rmsnorm_f32(const void *x_f32, size_t ldx, size_t rows, size_t cols, int groups, const void *w_bf16, float eps, int accumulate,
+                          void *y_f32, size_t ldy, ifa_stream stream);
+/* y = x + conv(x): causal convolution over time on each channel WITHOUT activation (w bf16 [channels][taps], last tap = current token),
+ * the last taps - 1 inputs carried in the slot like ifa_shortconv_silu_f32's (ifa_shortconv_tail_f32 advances them afterwards) */
+int ifa_shortconv_residual_f32(const void *x_f32, size_t ldx, int channels, int taps, const void *w_bf16, const void *seqs_dev, const int *row_seq_dev,
+                               size_t rows, void *const *slot_base_dev, size_t state_off, void *y_f32, size_t ldy, ifa_stream stream);
+/* depth average: stack[count - 1] <- x (rows x cols, contiguous), then x <- sum_j w[j] stack[j], j < count; stack planes are
+ * plane_stride floats apart; w bf16 [count] */
+int ifa_depth_average_f32(void *x_f32, size_t rows, size_t cols, void *stack_f32, size_t plane_stride, int count, const void *w_bf16, ifa_stream stream);
+/* x <- cap * tanh(x / cap) over n contiguous values */
+int ifa_softcap_f32(void *x_f32, size_t n, float cap, ifa_stream stream);
+
+/* ---- latent attention (csrc/ifa_attn_latent.hip): the cache of a layer holds ONE row per position, [kv_rank latent | rot_dim rotated key
+ * part] fp32, shared by all heads; keys and values of a head are linear maps of the latent (w_uk [heads * dim][kv_rank],
+ * w_uv [heads * vdim][kv_rank], bf16).  A query head is [dim unrotated | rot_dim rotated]; score = (q_u . W_uk c + q_r . k_r) * scale.
+ * Rotation: interleaved pairs (2i, 2i + 1) of the first rot_dims dimensions of the rotated part by angle pos * freq[i]
+ * (freq_f64_dev: double [rot_dims / 2], angles formed in double), cos and sin multiplied by rot_mult. */
+/* rows of a step: c = rms(kv[:kv_rank]) * c_norm_w and the rotated key part into the cache; the rotated part of every query head in place */
+int ifa_latent_prepare_f32(const void *kv_f32, size_t ldkv, int kv_rank, int rot_dim, int rot_dims, const void *c_norm_w_bf16, float eps,
+                           void *q_f32, size_t ldq, int heads, int dim, const double *freq_f64_dev, float rot_mult, const void *seqs_dev,
+                           const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t cache_off, ifa_stream stream);
+/* absorbed query: qa[t][h] = [W_uk[h]^T q_u[t][h] (kv_rank) | q_r[t][h] (rot_dim)]: a query against the cache rows themselves */
+int ifa_latent_absorb_q_f32(const void *q_f32, size_t ldq, int heads, int dim, int rot_dim, int kv_rank, const void *w_uk_bf16, size_t rows,
+                            void *qa_f32, size_t ldqa, ifa_stream stream);
+/* out[t][h * vdim + e] = gate[t][h] * sum_r w_uv[h * vdim + e][r] * ol[t][h * ld_head + r]; gate = sigmoid(g[t][h]) or 1 (g null) */
+int ifa_latent_expand_out_f32(const void *ol_f32, size_t ldol, int ld_head, int heads, int vdim, int kv_rank, const void *w_uv_bf16,
+                              const void *g_f32, size_t ldg, size_t rows, void *out_f32, size_t ldo, ifa_stream stream);
+/* prompts: causal softmax attention of the step's rows with per-head keys [kx (dim, expanded: kx_f32 [ctx rows][heads * dim]) | rotated
+ * part from the cache rows] and values vx_f32 [ctx rows][heads * vdim]; ctx0_dev[s] / seqs_host: first expanded row of sequence s (its
+ * position 0).  128 queries of one sequence per workgroup on the fp32 matrix cores, online softmax in fp32. */
+int ifa_attention_latent_tile_f32(const void *q_f32, size_t ldq, int heads, int dim, int rot_dim, int vdim, int kv_rank, float scale,
+                                  const void *kx_f32, size_t ldkx, const void *vx_f32, size_t ldvx, const int *ctx0_dev, const void *g_f32, size_t ldg,
+                                  const void *seqs_dev, const void *seqs_host, int n_seqs, void *const *slot_base_dev, size_t cache_off,
+                                  void *out_f32, size_t ldo, ifa_stream stream);
+/* 1 if the tiled kernel serves these head sizes (keys up to 192, values up to 128 dimensions, within the LDS) */
+int ifa_attention_latent_tile_fits(int dim, int rot_dim, int vdim);
+
+/* ---- mixture of experts (csrc/ifa_moe_f32.hip): `experts` feed-forward experts down(act(up h)) without biases (up bf16
+ * [experts][ff][width], down bf16 [experts][width][ff]) + `identity` experts whose output is h itself.  Router: scores = softmax of the
+ * logits over experts + identity; the `top` largest (score + correction) are chosen (lowest index on ties); weights = their scores,
+ * not renormalized.  idx_dev / wgt_dev: [rows][top]. */
+int ifa_moe_route_f32(const void *logits_f32, size_t ld, size_t rows, int n_all, int top, const void *correction_bf16, int *idx_dev, void *wgt_f32,
+                      ifa_stream stream);
+/* y[t] (+)= sum_k wgt[t][k] * expert_{idx[t][k]}(h[t]); act 0: exact (erf) GELU.  Rows are served by expert: few rows stream each chosen
+ * expert's weights per row; many rows are sorted by expert and run as grouped matrix-core products (ops32 as in ifa_linear_bf16w).
+ * ws: workspace of ifa_moe_workspace_bytes(rows, top, width, ff, experts) bytes.  Deterministic: no atomics on values. */
+size_t ifa_moe_workspace_bytes(size_t rows, int top, int width, int ff, int experts);
+int ifa_moe_experts_f32(const void *h_f32, size_t ldh, size_t rows, int width, int ff, int experts, int identity, int top, int act,
+                        const void *up_bf16, const void *down_bf16, const int *idx_dev, const void *wgt_f32, int ops32, void *ws, size_t ws_bytes,
+                        void *y_f32, size_t ldy, int accumulate, ifa_stream stream);
+
 /* ======================================================================== */
 /* Layer-list worker: a decoder whose layers are given one by one, each with its own sequence mixer, a 32-bit residual       */
 /* stream and bfloat16 weights (csrc/ifa_engine_layered.hip).  It is an ifa_model: finalize / kv_slots / select_kv /        */
@@ -531,7 +593,14 @@ int ifa_attention_window_f32(const void *q_f32, size_t ldq, int heads, int kv_he
 /* A layer: h = norm1(x); x <- x + ls1 * mixer(h) + ls2 * ffn(h)  (one norm, both sub-layers read it).                      */
 /* ======================================================================== */
 enum { IFA_MIX_WINDOW_LINEAR = 1,   /* windowed softmax attention (values = keys as projected) + decayed linear attention, side by side */
-       IFA_MIX_GATED_DELTA = 2 };   /* gated delta rule behind short convolutions */
+       IFA_MIX_GATED_DELTA = 2,     /* gated delta rule behind short convolutions */
+       IFA_MIX_LATENT = 3 };        /* latent attention: one compressed key / value row per position, a rotated key part shared by all heads */
+/* wiring of a layer.  PARALLEL: h = norm1(x); x <- x + ls1 * mixer(h) + ls2 * ffn(h).  POSTNORM: the sub-layers read x itself (plus a
+ * short causal convolution of x when canon_taps > 0) and the grouped RMS norm sits on their OUTPUT: x <- x + norm1(mixer(x'));
+ * x <- x + norm2(ffn(x')); with depth_avg the next layer reads sum_j dwa[j] X_j over the embedding output X_0 and every layer result. */
+enum { IFA_BLOCK_PARALLEL = 0, IFA_BLOCK_POSTNORM = 1 };
+enum { IFA_FFN_GATED = 0,           /* gated feed-forward (GELU tanh, biases), width `ffn` */
+       IFA_FFN_MOE = 1 };           /* mixture of experts: x_experts experts of width x_ff + x_identity identity experts, x_top per token */
 typedef struct {
     int mixer;                       /* IFA_MIX_* */
     int ffn;                         /* width of the gated feed-forward (GELU tanh, biases); 0 = none */
@@ -543,11 +612,24 @@ typedef struct {
     float l_out_scale;
     /* gated delta rule */
     int d_heads, d_kv_heads, d_dim, d_vdim, d_conv;
+    /* wiring (IFA_BLOCK_*), taps of the input convolution of both sub-layers (0: none), depth average on / off */
+    int block, canon_taps, depth_avg;
+    /* latent attention: heads of [m_dim unrotated | m_rot_dim rotated] query / key dimensions, values of m_vdim, latent of m_kv_rank;
+     * m_q_rank > 0: the queries go through an RMS-normed latent of that size; m_gate: a sigmoid gate per head on the output;
+     * the first m_rot_dims dimensions of the rotated part turn with base m_rot_base; m_yarn_factor > 0: YaRN frequency scaling */
+    int m_heads, m_dim, m_rot_dim, m_vdim, m_kv_rank, m_q_rank, m_gate, m_rot_dims;
+    float m_scale, m_rot_base, m_yarn_factor, m_yarn_original, m_yarn_fast, m_yarn_slow;
+    /* feed-forward kind (IFA_FFN_*) and the mixture's sizes */
+    int ffn_kind, x_experts, x_identity, x_top, x_ff;
 } ifa_layer_spec;
 typedef struct {
     int width, vocab, max_ctx, n_layers, device;
     int ops32;                       /* 1: matrix products keep fp32 operands (exact mode); 0: operands rounded to bfloat16 */
     float eps, pos_base;             /* eps of every norm of the stack; base of the sinusoidal position vector (10000) */
+    int stem;                        /* 0: embedding + sinusoidal position vector, layer norm before lm_head; 1: embedding through a grouped RMS
+                                      * norm (IFA_T_EMBD_NORM), grouped RMS norm before lm_head, no position vector */
+    int norm_groups;                 /* parts of the grouped RMS norms (stem 1 and POSTNORM layers) */
+    float logit_softcap;             /* > 0: logits <- cap * tanh(logits / cap) */
 } ifa_layered_config;
 /* tensors of a layer-list model (global ones use IFA_T_EMBD / IFA_T_OUT_NORM / IFA_T_LM_HEAD with layer = -1) */
 enum {
@@ -555,7 +637,10 @@ enum {
     IFA_LT_A_Q, IFA_LT_A_K, IFA_LT_A_REL, IFA_LT_A_SINK, IFA_LT_A_O,
     IFA_LT_L_Q, IFA_LT_L_K, IFA_LT_L_V, IFA_LT_L_G, IFA_LT_L_O, IFA_LT_L_NORM, IFA_LT_L_DECAY /* fp32 [heads] */,
     IFA_LT_D_Q, IFA_LT_D_K, IFA_LT_D_V, IFA_LT_D_QCONV, IFA_LT_D_KCONV, IFA_LT_D_VCONV, IFA_LT_D_B, IFA_LT_D_A, IFA_LT_D_ALOG, IFA_LT_D_DTBIAS,
-    IFA_LT_D_G, IFA_LT_D_NORM, IFA_LT_D_O, IFA_LT_END
+    IFA_LT_D_G, IFA_LT_D_NORM, IFA_LT_D_O,
+    IFA_LT_NORM2, IFA_LT_CANON1, IFA_LT_CANON2, IFA_LT_DWA,
+    IFA_LT_M_Q, IFA_LT_M_DQ, IFA_LT_M_DQ_NORM, IFA_LT_M_UQ, IFA_LT_M_DKV, IFA_LT_M_DKV_NORM, IFA_LT_M_UK, IFA_LT_M_UV, IFA_LT_M_G, IFA_LT_M_O,
+    IFA_LT_X_ROUTER, IFA_LT_X_CORR, IFA_LT_X_UP /* [experts * ff][width] */, IFA_LT_X_DOWN /* [experts * width][ff] */, IFA_LT_END
 };
 int ifa_model_create_layered(const ifa_layered_config *cfg, const ifa_layer_spec *layers, ifa_model **out);
 /* a tensor from HOST memory: dtype IFA_BF16 (bit patterns) or IFA_F32 (IFA_LT_L_DECAY only); shapes are checked against the specs */

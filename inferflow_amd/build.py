@@ -162,7 +162,8 @@ def build_library(force=False, verbose=False, jobs=None):
 # ---- profile "layered": a library with the layer-list worker class only (what bin/trace_run builds in a fresh checkout)
 LAYERED_LIB_PATH = os.path.join(LIB_DIR, "libinferflow_amd_layered.so")
 LAYERED_CLI_PATH = os.path.join(BIN_DIR, "ifa_trace_run_layered")
-LAYERED_UNITS = ["ifa_runtime.hip", "ifa_linear_bf16.hip", "ifa_ops_f32.hip", "ifa_seqmix.hip", "ifa_attn_window.hip", "ifa_engine_layered.hip",
+LAYERED_UNITS = ["ifa_runtime.hip", "ifa_linear_bf16.hip", "ifa_ops_f32.hip", "ifa_seqmix.hip", "ifa_attn_window.hip", "ifa_attn_latent.hip", "ifa_moe_f32.hip",
+                 "ifa_engine_layered.hip",
                  os.path.join("profile_layered", "ifa_model_api.hip")]
 
 
@@ -176,7 +177,7 @@ def layered_is_stale():
 
 
 def build_layered_library(force=False):
-    """libinferflow_amd_layered.so + bin/ifa_trace_run_layered: seven HIP units and the host engine (seconds, not minutes)."""
+    """libinferflow_amd_layered.so + bin/ifa_trace_run_layered: nine HIP units and the host engine (seconds, not minutes)."""
     if not force and not layered_is_stale():
         return LAYERED_LIB_PATH
     hipcc = _hipcc()

@@ -47,11 +47,12 @@ struct WinAttnArgs {
     float *ws; int nsplit;           // nsplit > 1: the keys of a (row, head) are shared out to nsplit workgroups; partial results in ws [rows][heads][nsplit][dim + 2]
 };
 
-constexpr int WA_DPL = 4;         // dim <= 64 * WA_DPL
+constexpr int WA_DPL_MAX = 10;    // dim <= 64 * DPL: a lane holds DPL value columns (1, 2, 4 or 10: up to 640, the row of a latent-attention cache)
 
 // grid (rows, heads, splits), four waves: the visible keys (kept first tokens, then the window) are walked in chunks of 16, four
 // lanes per key for the score, one value column per lane for the weighted sum; chunks go round-robin to the waves, each
 // with its own running maximum / sum / accumulator, merged through LDS at the end together with the sink.
+template <int WA_DPL>
 __global__ void __launch_bounds__(256) k_attn_window(WinAttnArgs P)
 {
     extern __shared__ float sm[];
@@ -329,7 +330,7 @@ int ifa_attention_window_f32(const void *q_f32, size_t ldq, int heads, int kv_he
 {
     IFA_REQUIRE(q_f32 && seqs_dev && row_seq_dev && slot_base_dev && out_f32, "ifa_attention_window_f32: null pointer");
     IFA_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && dim > 0 && rows > 0 && window >= 1 && keep_first >= 0, "ifa_attention_window_f32: bad shape");
-    IFA_REQUIRE(dim <= 64 * WA_DPL, "ifa_attention_window_f32: head size %d above %d", dim, 64 * WA_DPL);
+    IFA_REQUIRE(dim <= 64 * WA_DPL_MAX, "ifa_attention_window_f32: head size %d above %d", dim, 64 * WA_DPL_MAX);
     IFA_REQUIRE(!rel_bf16 || (bucket_of_dev && n_buckets > 0), "ifa_attention_window_f32: a bias table needs its bucket map");
     WinAttnArgs P;
     P.q = (const float *)q_f32; P.ldq = ldq; P.heads = heads; P.kv_heads = kv_heads; P.dim = dim; P.norm_q = norm_q; P.eps = eps; P.scale = scale;
@@ -359,7 +360,11 @@ int ifa_attention_window_f32(const void *q_f32, size_t ldq, int heads, int kv_he
         while (nsplit > 1 && rows * (size_t)heads * nsplit * ((size_t)dim + 2) * 4 > ws_bytes) nsplit--;
     }
     P.ws = (float *)ws_f32; P.nsplit = nsplit;
-    hipLaunchKernelGGL(k_attn_window, dim3((unsigned)rows, (unsigned)heads, (unsigned)nsplit), dim3(256), smem, ifa_s(stream), P);
+    const dim3 grid_rows((unsigned)rows, (unsigned)heads, (unsigned)nsplit);
+    if (dim <= 64) hipLaunchKernelGGL(k_attn_window<1>, grid_rows, dim3(256), smem, ifa_s(stream), P);
+    else if (dim <= 128) hipLaunchKernelGGL(k_attn_window<2>, grid_rows, dim3(256), smem, ifa_s(stream), P);
+    else if (dim <= 256) hipLaunchKernelGGL(k_attn_window<4>, grid_rows, dim3(256), smem, ifa_s(stream), P);
+    else hipLaunchKernelGGL(k_attn_window<WA_DPL_MAX>, grid_rows, dim3(256), smem, ifa_s(stream), P);
     if (nsplit > 1) hipLaunchKernelGGL(k_attn_window_combine, dim3((unsigned)rows, (unsigned)heads), dim3(64), 0, ifa_s(stream), P);
     IFA_LAUNCH_CHECK();
     return IFA_OK;

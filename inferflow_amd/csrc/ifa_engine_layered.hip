@@ -15,6 +15,10 @@
 // Per layer: norm1 -> ONE product for every projection that reads it (mixer inputs, gates, FFN gate | up; biases in the
 // epilogue) -> mixer kernels -> output products that add into the fp32 residual with layer scale and branch scale
 // in their epilogue -> GELU-gated FFN the same way.
+// Layers wired IFA_BLOCK_POSTNORM read the residual itself through a short causal convolution (x' = x + conv(x), its last taps - 1
+// inputs in the slot), put a grouped RMS norm on each sub-layer's OUTPUT (x <- x + norm(sub(x'))), mix with latent attention (cache row
+// [latent | rotated key part] per position; single tokens take the absorbed form, prompts expanded keys / values and the tiled
+// kernel), feed forward through a mixture of experts, and hand the next layer a learned average over the depth of the stack.
 #include <algorithm>
 #include <cmath>
 #include <cstring>
@@ -39,6 +43,10 @@ struct LLayer {
     int *bucket_of = nullptr;                         // distance -> bias row
     // arena offsets (floats)
     size_t o_k = 0, o_v = 0, o_lin = 0, o_rec = 0, o_conv = 0;
+    // latent attention: column offsets of q (or its latent), [latent | key part] and the head gates in the fused product; cache and
+    // convolution tails in the arena; rotation frequencies (double, device) and the factor on cos / sin
+    size_t c_mq = 0, c_mkv = 0, c_mg = 0, o_c = 0, o_cv1 = 0, o_cv2 = 0;
+    double *freq = nullptr; float rot_mult = 1.0f;
     LTensor &T(int id) { return t[id - IFA_LT_NORM1]; }
     const LTensor &T(int id) const { return t[id - IFA_LT_NORM1]; }
 };
@@ -50,7 +58,7 @@ constexpr int MAX_SLOTS = 4096;
 struct LayeredNet {
     ifa_layered_config cfg;
     std::vector<LLayer> layers;
-    LTensor embd, out_norm, lm_head;
+    LTensor embd, out_norm, lm_head, embd_norm;
     size_t arena_floats = 0;
     std::vector<float *> slot_ptr;       // host copy of the table (null: not allocated yet)
     float **slot_base_dev = nullptr;
@@ -72,6 +80,12 @@ struct LayeredNet {
     float *attn_ws = nullptr; size_t attn_ws_bytes = 0;      // partial results of the windowed attention when a (row, head)'s keys are shared out
     int opt_attn_tile_min = 16;            // steps of at least this many rows run the windowed attention through the tiled kernel
     std::vector<ifa_seq_desc> seqs_host;   // the current step's sequences (the tiled attention's grid is sized from them)
+    // POSTNORM layers: two more mixer buffers, the planes of the depth average ([layers + 1][scratch_rows * width]), the router's choices,
+    // the experts' workspace, and -- prompts through latent attention -- keys / values expanded for every position of the step's sequences
+    float *m4 = nullptr, *m5 = nullptr, *stack = nullptr, *moe_wgt = nullptr, *kx = nullptr, *vx = nullptr;
+    int *moe_idx = nullptr, *ctx0_dev = nullptr; void *moe_ws = nullptr; size_t moe_ws_bytes = 0, expand_rows = 0, kx_max = 0, vx_max = 0, top_max = 0;
+    bool any_depth_avg = false, any_latent = false, any_moe = false, latent_tile_ok = true, step_expand = false;
+    std::vector<int> ctx0_host; size_t step_ctx_rows = 0;
     hipGraphExec_t step_exec = nullptr; hipGraph_t step_graph = nullptr; int step_slot = -1;
 };
 
@@ -87,13 +101,36 @@ void drop_step_graph(LayeredNet *n)
 }
 
 // rows x cols a tensor of this layer must have; false: the tensor does not belong to the layer's mixer
-bool expected_shape(const LayeredNet *n, const ifa_layer_spec &s, int id, size_t &r, size_t &c, bool &vec)
+bool has_moe(const ifa_layer_spec &s) { return s.ffn_kind == IFA_FFN_MOE && s.x_experts + s.x_identity > 0; }
+
+bool expected_shape(const LayeredNet *n, const ifa_layer_spec &s, int li, int id, size_t &r, size_t &c, bool &vec)
 {
     const size_t W = (size_t)n->cfg.width;
     vec = false;
-    const bool par = s.mixer == IFA_MIX_WINDOW_LINEAR, del = s.mixer == IFA_MIX_GATED_DELTA;
+    const bool par = s.mixer == IFA_MIX_WINDOW_LINEAR, del = s.mixer == IFA_MIX_GATED_DELTA, lat = s.mixer == IFA_MIX_LATENT;
+    const bool post = s.block == IFA_BLOCK_POSTNORM, moe = has_moe(s);
+    const size_t MH = (size_t)s.m_heads, MQ = MH * (size_t)(s.m_dim + s.m_rot_dim), MR = (size_t)s.m_kv_rank, XA = (size_t)(s.x_experts + s.x_identity);
     switch (id) {
-    case IFA_LT_NORM1: case IFA_LT_LS1: r = 1; c = W; vec = true; return true;
+    case IFA_LT_NORM1: r = 1; c = W; vec = true; return true;
+    case IFA_LT_LS1: r = 1; c = W; vec = true; return !post;
+    case IFA_LT_NORM2: r = 1; c = W; vec = true; return post && moe;
+    case IFA_LT_CANON1: r = W; c = (size_t)s.canon_taps; return post && s.canon_taps > 0;
+    case IFA_LT_CANON2: r = W; c = (size_t)s.canon_taps; return post && s.canon_taps > 0 && moe;
+    case IFA_LT_DWA: r = 1; c = (size_t)li + 2; vec = true; return post && s.depth_avg;
+    case IFA_LT_M_Q: r = MQ; c = W; return lat && s.m_q_rank == 0;
+    case IFA_LT_M_DQ: r = (size_t)s.m_q_rank; c = W; return lat && s.m_q_rank > 0;
+    case IFA_LT_M_DQ_NORM: r = 1; c = (size_t)s.m_q_rank; vec = true; return lat && s.m_q_rank > 0;
+    case IFA_LT_M_UQ: r = MQ; c = (size_t)s.m_q_rank; return lat && s.m_q_rank > 0;
+    case IFA_LT_M_DKV: r = MR + (size_t)s.m_rot_dim; c = W; return lat;
+    case IFA_LT_M_DKV_NORM: r = 1; c = MR; vec = true; return lat;
+    case IFA_LT_M_UK: r = MH * (size_t)s.m_dim; c = MR; return lat;
+    case IFA_LT_M_UV: r = MH * (size_t)s.m_vdim; c = MR; return lat;
+    case IFA_LT_M_G: r = MH; c = W; return lat && s.m_gate;
+    case IFA_LT_M_O: r = W; c = MH * (size_t)s.m_vdim; return lat;
+    case IFA_LT_X_ROUTER: r = XA; c = W; return moe;
+    case IFA_LT_X_CORR: r = 1; c = XA; vec = true; return moe;
+    case IFA_LT_X_UP: r = (size_t)s.x_experts * s.x_ff; c = W; return moe && s.x_experts > 0;
+    case IFA_LT_X_DOWN: r = (size_t)s.x_experts * W; c = (size_t)s.x_ff; return moe && s.x_experts > 0;
     case IFA_LT_LS2: case IFA_LT_FFN_DOWN_B: r = 1; c = W; vec = true; return s.ffn > 0;
     case IFA_LT_FFN_GATE: case IFA_LT_FFN_UP: r = (size_t)s.ffn; c = W; return s.ffn > 0;
     case IFA_LT_FFN_GATE_B: case IFA_LT_FFN_UP_B: r = 1; c = (size_t)s.ffn; vec = true; return s.ffn > 0;
@@ -162,11 +199,12 @@ int ensure_rows(ifa_model *m, size_t T, size_t nseq)
         lay_free(n->tab_dev);
         n->tab_pin = nullptr; n->tab_dev = nullptr;
         const size_t R = std::max(T, n->tab_rows), S = std::max(nseq, n->tab_seqs);
-        const size_t ints = 3 * R + 4 * S;
+        const size_t ints = 3 * R + 5 * S;
         IFA_HIP_CHECK(hipHostMalloc((void **)&n->tab_pin, ints * 4, hipHostMallocDefault));
         IFA_HIP_CHECK(hipMalloc((void **)&n->tab_dev, ints * 4));
         n->tab_rows = R; n->tab_seqs = S;
         n->tokens_dev = n->tab_dev; n->pos_dev = n->tab_dev + R; n->row_seq_dev = n->tab_dev + 2 * R; n->seqs_dev = (ifa_seq_desc *)(n->tab_dev + 3 * R);
+        n->ctx0_dev = n->tab_dev + 3 * R + 4 * S;
     }
     if (T > n->scratch_rows) {
         IFA_HIP_CHECK(hipStreamSynchronize(m->stream));
@@ -176,6 +214,17 @@ int ensure_rows(ifa_model *m, size_t T, size_t nseq)
         const size_t W = (size_t)n->cfg.width;
         const size_t sz[] = {W, W, n->n_in_max, n->mix_max, n->mix_max, std::max<size_t>(n->ffn_max, 4), std::max<size_t>(n->heads_max, 4), std::max<size_t>(n->heads_max, 4)};
         for (size_t i = 0; i < 8; i++) IFA_HIP_CHECK(hipMalloc((void **)bufs[i], T * sz[i] * 4));
+        lay_free(n->m4); lay_free(n->m5); lay_free(n->stack); lay_free(n->moe_wgt); lay_free(n->moe_idx); lay_free(n->moe_ws);
+        n->m4 = n->m5 = n->stack = n->moe_wgt = nullptr; n->moe_idx = nullptr; n->moe_ws = nullptr; n->moe_ws_bytes = 0;
+        if (n->any_latent) { IFA_HIP_CHECK(hipMalloc((void **)&n->m4, T * n->mix_max * 4)); IFA_HIP_CHECK(hipMalloc((void **)&n->m5, T * n->mix_max * 4)); }
+        if (n->any_depth_avg) IFA_HIP_CHECK(hipMalloc((void **)&n->stack, (n->layers.size() + 1) * T * W * 4));
+        if (n->any_moe) {
+            IFA_HIP_CHECK(hipMalloc((void **)&n->moe_wgt, T * n->top_max * 4));
+            IFA_HIP_CHECK(hipMalloc((void **)&n->moe_idx, T * n->top_max * 4));
+            for (const LLayer &L : n->layers)
+                if (has_moe(L.spec)) n->moe_ws_bytes = std::max(n->moe_ws_bytes, ifa_moe_workspace_bytes(T, L.spec.x_top, (int)W, std::max(L.spec.x_ff, 1), L.spec.x_experts));
+            IFA_HIP_CHECK(hipMalloc(&n->moe_ws, n->moe_ws_bytes));
+        }
         n->scratch_rows = T;
     }
     return IFA_OK;
@@ -200,6 +249,77 @@ int linear(ifa_model *m, const bf16_t *W, size_t N, size_t K, const float *A, si
     return ifa_linear_bf16w(W, N, K, A, lda, T, bias, mul, alpha, accumulate, m->lay->cfg.ops32, C, ldc, silu0, silu1, (ifa_stream)m->stream);
 }
 
+// one POSTNORM layer over T rows: x <- x + norm1(mixer(x + conv1(x))); x <- x + norm2(experts(x + conv2(x)))
+int run_postnorm_layer(ifa_model *m, LLayer &L, size_t li, size_t T, int nseq)
+{
+    LayeredNet *n = m->lay;
+    const ifa_layered_config &c = n->cfg;
+    const ifa_layer_spec &sp = L.spec;
+    const size_t W = (size_t)c.width, NI = L.n_in;
+    ifa_stream s = (ifa_stream)m->stream;
+    void *const *slots = (void *const *)n->slot_base_dev;
+    int rc;
+    // what the mixer reads
+    const float *hin = n->x;
+    if (sp.canon_taps > 0) {
+        if ((rc = ifa_shortconv_residual_f32(n->x, W, (int)W, sp.canon_taps, L.T(IFA_LT_CANON1).data, n->seqs_dev, n->row_seq_dev, T, slots, L.o_cv1, n->h, W, s))) return rc;
+        if ((rc = ifa_shortconv_tail_f32(n->x, W, (int)W, sp.canon_taps, n->seqs_dev, nseq, slots, L.o_cv1, s))) return rc;
+        hin = n->h;
+    }
+    {   // latent attention
+        const int H = sp.m_heads, dn = sp.m_dim, dr = sp.m_rot_dim, dv = sp.m_vdim, R = sp.m_kv_rank;
+        const size_t QD = (size_t)H * (dn + dr), CR = (size_t)(R + dr), OV = (size_t)H * dv;
+        if ((rc = linear(m, L.w_in, NI, W, hin, W, T, nullptr, nullptr, 1.0f, 0, n->proj, NI))) return rc;
+        float *q = n->proj + L.c_mq; size_t ldq = NI;
+        if (sp.m_q_rank > 0) {      // queries through their own normed latent
+            const size_t QR = (size_t)sp.m_q_rank;
+            if ((rc = ifa_layernorm_f32(0, n->proj + L.c_mq, NI, T, QR, L.T(IFA_LT_M_DQ_NORM).data, c.eps, n->m3, QR, s))) return rc;
+            if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_M_UQ).data, QD, QR, n->m3, QR, T, nullptr, nullptr, 1.0f, 0, n->m1, QD))) return rc;
+            q = n->m1; ldq = QD;
+        }
+        if ((rc = ifa_latent_prepare_f32(n->proj + L.c_mkv, NI, R, dr, sp.m_rot_dims, L.T(IFA_LT_M_DKV_NORM).data, c.eps, q, ldq, H, dn, L.freq, L.rot_mult,
+                                         n->seqs_dev, n->row_seq_dev, T, slots, L.o_c, s))) return rc;
+        const float *gate = sp.m_gate ? n->proj + L.c_mg : nullptr;
+        if (n->step_expand) {
+            // keys and values of every position of the step's sequences from their cached latents, then the tiled kernel
+            const size_t ldk = (size_t)H * dn, ldv = OV;
+            for (size_t qi = 0; qi < n->seqs_host.size(); qi++) {
+                const ifa_seq_desc &sd = n->seqs_host[qi];
+                const float *lat = n->slot_ptr[(size_t)sd.slot] + L.o_c;
+                const size_t ctx = (size_t)sd.pos0 + sd.n, r0 = (size_t)n->ctx0_host[qi];
+                if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_M_UK).data, ldk, (size_t)R, lat, CR, ctx, nullptr, nullptr, 1.0f, 0, n->kx + r0 * ldk, ldk))) return rc;
+                if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_M_UV).data, ldv, (size_t)R, lat, CR, ctx, nullptr, nullptr, 1.0f, 0, n->vx + r0 * ldv, ldv))) return rc;
+            }
+            if ((rc = ifa_attention_latent_tile_f32(q, ldq, H, dn, dr, dv, R, sp.m_scale, n->kx, ldk, n->vx, ldv, n->ctx0_dev, gate, NI, n->seqs_dev, n->seqs_host.data(),
+                                                    (int)n->seqs_host.size(), slots, L.o_c, n->m5, OV, s))) return rc;
+        } else {
+            // absorbed form: the cache rows are keys and values of ONE shared head of kv_rank + rot_dim dimensions
+            const size_t QA = (size_t)H * CR;
+            if ((rc = ifa_latent_absorb_q_f32(q, ldq, H, dn, dr, R, L.T(IFA_LT_M_UK).data, T, n->m2, QA, s))) return rc;
+            if ((rc = ifa_attention_window_f32(n->m2, QA, H, 1, (int)CR, 0, c.eps, sp.m_scale, 0.0f, c.max_ctx, 0, nullptr, nullptr, 0, nullptr, n->seqs_dev, n->row_seq_dev,
+                                               T, slots, L.o_c, L.o_c, n->m4, QA, nullptr, 0, 1 << 30, n->attn_ws, n->attn_ws_bytes, s))) return rc;
+            if ((rc = ifa_latent_expand_out_f32(n->m4, QA, (int)CR, H, dv, R, L.T(IFA_LT_M_UV).data, gate, NI, T, n->m5, OV, s))) return rc;
+        }
+        if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_M_O).data, W, OV, n->m5, OV, T, nullptr, nullptr, 1.0f, 0, n->m1, W))) return rc;
+        if ((rc = ifa_group_rmsnorm_f32(n->m1, W, T, W, c.norm_groups, L.T(IFA_LT_NORM1).data, c.eps, 1, n->x, W, s))) return rc;
+    }
+    if (has_moe(sp)) {
+        hin = n->x;
+        if (sp.canon_taps > 0) {
+            if ((rc = ifa_shortconv_residual_f32(n->x, W, (int)W, sp.canon_taps, L.T(IFA_LT_CANON2).data, n->seqs_dev, n->row_seq_dev, T, slots, L.o_cv2, n->h, W, s))) return rc;
+            if ((rc = ifa_shortconv_tail_f32(n->x, W, (int)W, sp.canon_taps, n->seqs_dev, nseq, slots, L.o_cv2, s))) return rc;
+            hin = n->h;
+        }
+        const size_t XA = (size_t)(sp.x_experts + sp.x_identity);
+        if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_X_ROUTER).data, XA, W, hin, W, T, nullptr, nullptr, 1.0f, 0, n->m2, XA))) return rc;
+        if ((rc = ifa_moe_route_f32(n->m2, XA, T, (int)XA, sp.x_top, L.T(IFA_LT_X_CORR).data, n->moe_idx, n->moe_wgt, s))) return rc;
+        if ((rc = ifa_moe_experts_f32(hin, W, T, (int)W, std::max(sp.x_ff, 1), sp.x_experts, sp.x_identity, sp.x_top, 0, L.T(IFA_LT_X_UP).data, L.T(IFA_LT_X_DOWN).data,
+                                      n->moe_idx, n->moe_wgt, c.ops32, n->moe_ws, n->moe_ws_bytes, n->m1, W, 0, s))) return rc;
+        if ((rc = ifa_group_rmsnorm_f32(n->m1, W, T, W, c.norm_groups, L.T(IFA_LT_NORM2).data, c.eps, 1, n->x, W, s))) return rc;
+    }
+    return IFA_OK;
+}
+
 // the layers of one step over T rows / nseq sequences whose tables are already on the device; leaves the residual in n->x
 int run_layers(ifa_model *m, size_t T, int nseq)
 {
@@ -209,10 +329,22 @@ int run_layers(ifa_model *m, size_t T, int nseq)
     ifa_stream s = (ifa_stream)m->stream;
     void *const *slots = (void *const *)n->slot_base_dev;
     int rc;
-    if ((rc = ifa_embed_sinpos_f32(n->embd.data, c.vocab, c.width, n->tokens_dev, n->pos_dev, T, c.pos_base, n->x, s))) return rc;
+    const size_t plane = n->scratch_rows * W;          // one plane of the depth average
+    if (c.stem == 1) {
+        if ((rc = ifa_embed_rows_f32(n->embd.data, c.vocab, c.width, n->tokens_dev, T, n->h, s))) return rc;
+        if ((rc = ifa_group_rmsnorm_f32(n->h, W, T, W, c.norm_groups, n->embd_norm.data, c.eps, 0, n->x, W, s))) return rc;
+        if (n->any_depth_avg && (rc = ifa_group_rmsnorm_f32(n->h, W, T, W, c.norm_groups, n->embd_norm.data, c.eps, 0, n->stack, W, s))) return rc;      // plane 0
+    } else if ((rc = ifa_embed_sinpos_f32(n->embd.data, c.vocab, c.width, n->tokens_dev, n->pos_dev, T, c.pos_base, n->x, s))) return rc;
     for (size_t li = 0; li < n->layers.size(); li++) {
         LLayer &L = n->layers[li];
         const ifa_layer_spec &sp = L.spec;
+        if (sp.block == IFA_BLOCK_POSTNORM) {
+            if ((rc = run_postnorm_layer(m, L, li, T, nseq))) return rc;
+            if (sp.depth_avg && (rc = ifa_depth_average_f32(n->x, T, W, n->stack, plane, (int)li + 2, L.T(IFA_LT_DWA).data, s))) return rc;
+            if (n->opt_tap_layers && n->taps && T <= n->taps_rows)
+                IFA_HIP_CHECK(hipMemcpyAsync(n->taps + li * n->taps_rows * W, n->x, T * W * 4, hipMemcpyDeviceToDevice, m->stream));
+            continue;
+        }
         const bf16_t *ls1 = (const bf16_t *)L.T(IFA_LT_LS1).data;
         const size_t NI = L.n_in;
         // (the linear attention's q | k | v leave the product through SiLU: contiguous columns [c_lq, c_lg))
@@ -269,20 +401,30 @@ int run_layers(ifa_model *m, size_t T, int nseq)
     return IFA_OK;
 }
 
+// the norm in front of lm_head: layer norm without bias, or (stem 1) the grouped RMS norm
+int out_norm_rows(ifa_model *m, const float *src, size_t rows, float *dst)
+{
+    LayeredNet *n = m->lay;
+    const size_t W = (size_t)n->cfg.width;
+    if (n->cfg.stem == 1) return ifa_group_rmsnorm_f32(src, W, rows, W, n->cfg.norm_groups, n->out_norm.data, n->cfg.eps, 0, dst, W, (ifa_stream)m->stream);
+    return ifa_layernorm_f32(1, src, W, rows, W, n->out_norm.data, n->cfg.eps, dst, W, (ifa_stream)m->stream);
+}
+
 // final norm + lm_head over rows [r0, r0 + nr) of the residual -> n->logits rows [0, nr)
 int run_head(ifa_model *m, size_t r0, size_t nr)
 {
     LayeredNet *n = m->lay;
     const size_t W = (size_t)n->cfg.width, V = (size_t)n->cfg.vocab;
     int rc;
-    if ((n->opt_fuse_rows & 1) && nr <= 8 && W % 8 == 0) {
+    if ((n->opt_fuse_rows & 1) && nr <= 8 && W % 8 == 0 && n->cfg.stem == 0) {
         if ((rc = ifa_linear_bf16w_rows(1, n->out_norm.data, n->cfg.eps, n->lm_head.data, V, W, n->x + r0 * W, W, nr, nullptr, nullptr, 1.0f, 0, n->logits, V, 0, 0,
                                         (ifa_stream)m->stream))) return rc;
         n->logits_rows = nr;
         return IFA_OK;
     }
-    if ((rc = ifa_layernorm_f32(1, n->x + r0 * W, W, nr, W, n->out_norm.data, n->cfg.eps, n->h, W, (ifa_stream)m->stream))) return rc;
+    if ((rc = out_norm_rows(m, n->x + r0 * W, nr, n->h))) return rc;
     if ((rc = linear(m, (const bf16_t *)n->lm_head.data, V, W, n->h, W, nr, nullptr, nullptr, 1.0f, 0, n->logits, V))) return rc;
+    if (n->cfg.logit_softcap > 0.0f && (rc = ifa_softcap_f32(n->logits, nr * V, n->cfg.logit_softcap, (ifa_stream)m->stream))) return rc;
     n->logits_rows = nr;
     return IFA_OK;
 }
@@ -301,9 +443,10 @@ int lay_destroy(ifa_model *m)
     drop_step_graph(n);
     for (LLayer &L : n->layers) {
         for (LTensor &t : L.t) lay_free(t.data);
-        lay_free(L.w_in); lay_free(L.b_in); lay_free(L.w_conv); lay_free(L.bucket_of);
+        lay_free(L.w_in); lay_free(L.b_in); lay_free(L.w_conv); lay_free(L.bucket_of); lay_free(L.freq);
     }
-    lay_free(n->embd.data); lay_free(n->out_norm.data); lay_free(n->lm_head.data);
+    lay_free(n->embd.data); lay_free(n->out_norm.data); lay_free(n->lm_head.data); lay_free(n->embd_norm.data);
+    lay_free(n->m4); lay_free(n->m5); lay_free(n->stack); lay_free(n->moe_wgt); lay_free(n->moe_idx); lay_free(n->moe_ws); lay_free(n->kx); lay_free(n->vx);
     for (float *p : n->slot_ptr) lay_free(p);
     lay_free(n->slot_base_dev);
     if (n->tab_pin) (void)hipHostFree(n->tab_pin);
@@ -335,6 +478,7 @@ int lay_finalize(ifa_model *m)
     IFA_HIP_CHECK(hipSetDevice(m->cfg.device));
     const size_t W = (size_t)n->cfg.width;
     IFA_REQUIRE(n->embd.present() && n->out_norm.present() && n->lm_head.present(), "layer-list worker: embedding, final norm or lm_head is missing");
+    IFA_REQUIRE(n->cfg.stem != 1 || n->embd_norm.present(), "layer-list worker: the norm behind the embedding is missing");
     size_t off = 0;
     n->n_in_max = n->mix_max = n->ffn_max = n->heads_max = 4;
     for (size_t li = 0; li < n->layers.size(); li++) {
@@ -343,11 +487,48 @@ int lay_finalize(ifa_model *m)
         if (L.w_in) continue;          // finalized before
         for (int id = IFA_LT_NORM1; id < IFA_LT_END; id++) {
             size_t r, c; bool vec;
-            if (expected_shape(n, sp, id, r, c, vec)) IFA_REQUIRE(L.T(id).present(), "layer-list worker: tensor %d of layer %zu is missing", id, li);
+            if (expected_shape(n, sp, (int)li, id, r, c, vec)) IFA_REQUIRE(L.T(id).present(), "layer-list worker: tensor %d of layer %zu is missing", id, li);
         }
         std::vector<bf16_t> w, b;
         int rc;
-        if (sp.mixer == IFA_MIX_WINDOW_LINEAR) {
+        if (sp.mixer == IFA_MIX_LATENT) {
+            if ((rc = cat_rows(w, b, L.T(sp.m_q_rank > 0 ? IFA_LT_M_DQ : IFA_LT_M_Q), nullptr, W, L.c_mq, m->stream))
+                || (rc = cat_rows(w, b, L.T(IFA_LT_M_DKV), nullptr, W, L.c_mkv, m->stream))
+                || (sp.m_gate && (rc = cat_rows(w, b, L.T(IFA_LT_M_G), nullptr, W, L.c_mg, m->stream)))) return rc;
+            // rotation frequencies in double: base^(-2i / dims), YaRN: the scaled and the plain frequency blended by a ramp over i
+            const int half = sp.m_rot_dims / 2;
+            std::vector<double> fr((size_t)std::max(half, 1), 0.0);
+            L.rot_mult = 1.0f;
+            const double dims = (double)sp.m_rot_dims, base = (double)sp.m_rot_base;
+            for (int i = 0; i < half; i++) fr[(size_t)i] = std::pow(base, -2.0 * i / dims);
+            if (sp.m_yarn_factor > 0.0f) {
+                const double factor = sp.m_yarn_factor, orig = sp.m_yarn_original, two_pi = 6.283185307179586476925;
+                auto dim_of = [&](double turns) { return dims * std::log(orig / (two_pi * turns)) / (2.0 * std::log(base)); };
+                const double lo = std::max(std::floor(dim_of(sp.m_yarn_fast)), 0.0), hi = std::min(std::ceil(dim_of(sp.m_yarn_slow)), dims - 1.0);
+                for (int i = 0; i < half; i++) {
+                    const double ramp = std::min(1.0, std::max(0.0, ((double)i - lo) / std::max(hi - lo, 0.001)));
+                    fr[(size_t)i] = fr[(size_t)i] / factor * ramp + fr[(size_t)i] * (1.0 - ramp);
+                }
+                L.rot_mult = (float)(0.1 * std::log(factor) + 1.0);
+            }
+            IFA_HIP_CHECK(hipMalloc((void **)&L.freq, fr.size() * 8));
+            IFA_HIP_CHECK(hipMemcpy(L.freq, fr.data(), fr.size() * 8, hipMemcpyHostToDevice));
+            const size_t CR = (size_t)(sp.m_kv_rank + sp.m_rot_dim), H = (size_t)sp.m_heads;
+            L.o_c = off; off += align4((size_t)n->cfg.max_ctx * CR);
+            if (sp.canon_taps > 1) { L.o_cv1 = off; off += align4((size_t)(sp.canon_taps - 1) * W); }
+            n->mix_max = std::max({n->mix_max, H * (size_t)(sp.m_dim + sp.m_rot_dim), H * CR, H * (size_t)sp.m_vdim, W, (size_t)sp.m_q_rank});
+            n->ffn_max = std::max(n->ffn_max, (size_t)sp.m_q_rank);
+            n->kx_max = std::max(n->kx_max, H * (size_t)sp.m_dim); n->vx_max = std::max(n->vx_max, H * (size_t)sp.m_vdim);
+            n->any_latent = true;
+            if (!ifa_attention_latent_tile_fits(sp.m_dim, sp.m_rot_dim, sp.m_vdim)) n->latent_tile_ok = false;
+            if (has_moe(sp)) {
+                if (sp.canon_taps > 1) { L.o_cv2 = off; off += align4((size_t)(sp.canon_taps - 1) * W); }
+                n->mix_max = std::max(n->mix_max, (size_t)(sp.x_experts + sp.x_identity));
+                n->top_max = std::max(n->top_max, (size_t)sp.x_top);
+                n->any_moe = true;
+            }
+            if (sp.depth_avg) n->any_depth_avg = true;
+        } else if (sp.mixer == IFA_MIX_WINDOW_LINEAR) {
             if ((rc = cat_rows(w, b, L.T(IFA_LT_A_Q), nullptr, W, L.c_aq, m->stream)) || (rc = cat_rows(w, b, L.T(IFA_LT_A_K), nullptr, W, L.c_ak, m->stream))
                 || (rc = cat_rows(w, b, L.T(IFA_LT_L_Q), nullptr, W, L.c_lq, m->stream)) || (rc = cat_rows(w, b, L.T(IFA_LT_L_K), nullptr, W, L.c_lk, m->stream))
                 || (rc = cat_rows(w, b, L.T(IFA_LT_L_V), nullptr, W, L.c_lv, m->stream)) || (rc = cat_rows(w, b, L.T(IFA_LT_L_G), nullptr, W, L.c_lg, m->stream))) return rc;
@@ -394,7 +575,7 @@ int lay_finalize(ifa_model *m)
         n->n_in_max = std::max(n->n_in_max, L.n_in);
         // the separate copies of what the fused product now holds are no longer needed
         for (int id : {IFA_LT_A_Q, IFA_LT_A_K, IFA_LT_L_Q, IFA_LT_L_K, IFA_LT_L_V, IFA_LT_L_G, IFA_LT_D_Q, IFA_LT_D_K, IFA_LT_D_V, IFA_LT_D_B, IFA_LT_D_A,
-                       IFA_LT_D_G, IFA_LT_FFN_GATE, IFA_LT_FFN_UP}) {
+                       IFA_LT_D_G, IFA_LT_FFN_GATE, IFA_LT_FFN_UP, IFA_LT_M_Q, IFA_LT_M_DQ, IFA_LT_M_DKV, IFA_LT_M_G}) {
             LTensor &t = L.T(id);
             if (t.data) { lay_free(t.data); t.data = nullptr; }
         }
@@ -403,6 +584,7 @@ int lay_finalize(ifa_model *m)
         size_t per_row = 0;
         for (const LLayer &L : n->layers)
             if (L.spec.mixer == IFA_MIX_WINDOW_LINEAR) per_row = std::max(per_row, (size_t)L.spec.a_heads * 32 * ((size_t)L.spec.a_dim + 2) * 4);
+            else if (L.spec.mixer == IFA_MIX_LATENT) per_row = std::max(per_row, (size_t)L.spec.m_heads * 32 * ((size_t)(L.spec.m_kv_rank + L.spec.m_rot_dim) + 2) * 4);
         n->attn_ws_bytes = per_row * 64;
         if (n->attn_ws_bytes) IFA_HIP_CHECK(hipMalloc((void **)&n->attn_ws, n->attn_ws_bytes));
     }
@@ -490,7 +672,13 @@ int upload_tables(ifa_model *m, const std::vector<int> &tokens, const std::vecto
     memcpy(n->tab_pin + 2 * R, row_seq.data(), T * 4);
     memcpy(n->tab_pin + 3 * R, seqs.data(), S * sizeof(ifa_seq_desc));
     n->seqs_host = seqs;
-    IFA_HIP_CHECK(hipMemcpyAsync(n->tab_dev, n->tab_pin, (3 * R + 4 * S) * 4, hipMemcpyHostToDevice, m->stream));
+    // first row of every sequence in the expanded key / value scratch (its position 0), for steps that take the tiled latent attention
+    n->ctx0_host.assign(S, 0);
+    size_t ctx_rows = 0;
+    for (size_t q = 0; q < S; q++) { n->ctx0_host[q] = (int)ctx_rows; ctx_rows += (size_t)seqs[q].pos0 + seqs[q].n; }
+    n->step_ctx_rows = ctx_rows;
+    memcpy(n->tab_pin + 3 * R + 4 * n->tab_seqs, n->ctx0_host.data(), S * 4);
+    IFA_HIP_CHECK(hipMemcpyAsync(n->tab_dev, n->tab_pin, (3 * R + 4 * n->tab_seqs + S) * 4, hipMemcpyHostToDevice, m->stream));
     return IFA_OK;
 }
 
@@ -539,7 +727,22 @@ int lay_step(ifa_model *m, int nseq, const int *tokens_host, const int *lens, co
         for (int i = 0; i < lens[q]; i++, r++) { pos[r] = pos0[q] + i; rs[r] = q; }
         last[(size_t)q] = (int)r - 1;
     }
-    if ((rc = upload_tables(m, tok, pos, rs, sq)) || (rc = run_layers(m, T, nseq))) return rc;
+    if ((rc = upload_tables(m, tok, pos, rs, sq))) return rc;
+    // prompts through latent attention: expanded keys / values + the tiled kernel when a sequence brings enough rows
+    n->step_expand = false;
+    if (n->any_latent && n->latent_tile_ok) {
+        int longest = 0;
+        for (int q = 0; q < nseq; q++) longest = std::max(longest, lens[q]);
+        n->step_expand = longest >= n->opt_attn_tile_min;
+    }
+    if (n->step_expand && n->step_ctx_rows > n->expand_rows) {
+        IFA_HIP_CHECK(hipStreamSynchronize(m->stream));
+        lay_free(n->kx); lay_free(n->vx); n->kx = n->vx = nullptr;
+        IFA_HIP_CHECK(hipMalloc((void **)&n->kx, n->step_ctx_rows * n->kx_max * 4));
+        IFA_HIP_CHECK(hipMalloc((void **)&n->vx, n->step_ctx_rows * n->vx_max * 4));
+        n->expand_rows = n->step_ctx_rows;
+    }
+    if ((rc = run_layers(m, T, nseq))) return rc;
     ifa_stream s = (ifa_stream)m->stream;
     if (all) {
         if ((rc = run_head(m, 0, T))) return rc;
@@ -548,8 +751,9 @@ int lay_step(ifa_model *m, int nseq, const int *tokens_host, const int *lens, co
     } else {
         // the sequences' last rows, normed one by one into consecutive rows of h, then one product
         for (int q = 0; q < nseq; q++)
-            if ((rc = ifa_layernorm_f32(1, n->x + (size_t)last[(size_t)q] * W, W, 1, W, n->out_norm.data, n->cfg.eps, n->h + (size_t)q * W, W, s))) return rc;
+            if ((rc = out_norm_rows(m, n->x + (size_t)last[(size_t)q] * W, 1, n->h + (size_t)q * W))) return rc;
         if ((rc = linear(m, (const bf16_t *)n->lm_head.data, V, W, n->h, W, (size_t)nseq, nullptr, nullptr, 1.0f, 0, n->logits, V))) return rc;
+        if (n->cfg.logit_softcap > 0.0f && (rc = ifa_softcap_f32(n->logits, (size_t)nseq * V, n->cfg.logit_softcap, s))) return rc;
         n->logits_rows = (size_t)nseq;
         if ((rc = ifa_argmax_rows_f32(n->logits, V, V, (size_t)nseq, n->excl_dev, n->next_dev, s))) return rc;
     }
@@ -604,6 +808,7 @@ int lay_decode(ifa_model *m, int first_token, int start_pos, int n_steps, int *o
     if ((rc = check_span(m, n_steps, start_pos, nullptr)) || (rc = ensure_slot(m, n->cur_slot)) || (rc = ensure_rows(m, 1, 1)) || (rc = ensure_logits(m, 1))) return rc;
     if (n->opt_graph && !n->opt_tap_layers && !n->step_exec) {      // (the slot is read from the device tables: one capture serves every slot)
         drop_step_graph(n);
+        n->step_expand = false;
         IFA_HIP_CHECK(hipStreamSynchronize(m->stream));
         IFA_HIP_CHECK(hipStreamBeginCapture(m->stream, hipStreamCaptureModeThreadLocal));
         rc = enqueue_decode_step(m);
@@ -621,6 +826,7 @@ int lay_decode(ifa_model *m, int first_token, int start_pos, int n_steps, int *o
     std::vector<int> tok(1, first_token), pos(1, start_pos), rs(1, 0);
     std::vector<ifa_seq_desc> sq(1); sq[0] = ifa_seq_desc{0, 1, start_pos, n->cur_slot};
     if ((rc = upload_tables(m, tok, pos, rs, sq))) return rc;
+    n->step_expand = false;
     hipEvent_t e0 = nullptr, e1 = nullptr;
     if (elapsed_ms) { IFA_HIP_CHECK(hipEventCreate(&e0)); IFA_HIP_CHECK(hipEventCreate(&e1)); IFA_HIP_CHECK(hipEventRecord(e0, m->stream)); }
     for (int st = 0; st < n_steps; st++) {
@@ -657,8 +863,23 @@ int ifa_model_create_layered(const ifa_layered_config *cfg, const ifa_layer_spec
         } else if (s.mixer == IFA_MIX_GATED_DELTA) {
             IFA_REQUIRE(s.d_heads > 0 && s.d_kv_heads > 0 && s.d_heads % s.d_kv_heads == 0 && s.d_dim > 0 && s.d_dim <= 256 && s.d_vdim > 0 && s.d_conv >= 1 && s.d_conv <= 64,
                         "ifa_model_create_layered: layer %d: bad delta-rule sizes", l);
+        } else if (s.mixer == IFA_MIX_LATENT) {
+            IFA_REQUIRE(s.m_heads > 0 && s.m_dim > 0 && s.m_rot_dim >= 0 && s.m_vdim > 0 && s.m_kv_rank > 0 && s.m_q_rank >= 0 && s.m_kv_rank + s.m_rot_dim <= 640
+                        && s.m_rot_dims >= 0 && s.m_rot_dims <= s.m_rot_dim && s.m_rot_dims % 2 == 0 && (s.m_rot_dims == 0 || s.m_rot_base > 1.0f),
+                        "ifa_model_create_layered: layer %d: bad latent-attention sizes", l);
+            IFA_REQUIRE(s.m_yarn_factor == 0.0f || (s.m_yarn_factor > 0.0f && s.m_yarn_original > 0.0f && s.m_yarn_fast > 0.0f && s.m_yarn_slow > 0.0f),
+                        "ifa_model_create_layered: layer %d: bad frequency scaling", l);
         } else return ifa_fail(IFA_ERR_ARG, "ifa_model_create_layered: layer %d: unknown mixer %d", l, s.mixer);
+        IFA_REQUIRE((s.block == IFA_BLOCK_POSTNORM) == (s.mixer == IFA_MIX_LATENT), "ifa_model_create_layered: layer %d: mixer %d is not wired for block kind %d", l, s.mixer, s.block);
+        if (s.block == IFA_BLOCK_POSTNORM) {
+            IFA_REQUIRE(s.ffn == 0 && s.canon_taps >= 0 && s.canon_taps <= 64 && cfg->norm_groups >= 1 && cfg->width % cfg->norm_groups == 0,
+                        "ifa_model_create_layered: layer %d: bad block sizes (norm in %d parts of width %d)", l, cfg->norm_groups, cfg->width);
+            if (s.ffn_kind == IFA_FFN_MOE && s.x_experts + s.x_identity > 0)
+                IFA_REQUIRE(s.x_experts >= 0 && s.x_identity >= 0 && s.x_experts + s.x_identity <= 4096 && s.x_top >= 1 && s.x_top <= s.x_experts + s.x_identity
+                            && (s.x_experts == 0 || s.x_ff > 0), "ifa_model_create_layered: layer %d: bad mixture-of-experts sizes", l);
+        } else IFA_REQUIRE(s.ffn_kind == IFA_FFN_GATED, "ifa_model_create_layered: layer %d: the mixture of experts needs the post-norm wiring", l);
     }
+    IFA_REQUIRE(cfg->stem == 0 || (cfg->stem == 1 && cfg->norm_groups >= 1 && cfg->width % cfg->norm_groups == 0), "ifa_model_create_layered: bad stem");
     IFA_HIP_CHECK(hipSetDevice(cfg->device));
     ifa_model *m = new ifa_model();
     memset(&m->cfg, 0, sizeof(m->cfg));
@@ -690,11 +911,12 @@ int ifa_model_set_tensor_host(ifa_model *m, int layer, int tensor_id, int dtype,
         if (tensor_id == IFA_T_EMBD) { t = &n->embd; er = V; ec = W; }
         else if (tensor_id == IFA_T_LM_HEAD) { t = &n->lm_head; er = V; ec = W; }
         else if (tensor_id == IFA_T_OUT_NORM) { t = &n->out_norm; er = 1; ec = W; vec = true; }
+        else if (tensor_id == IFA_T_EMBD_NORM) { t = &n->embd_norm; er = 1; ec = W; vec = true; }
         else return ifa_fail(IFA_ERR_ARG, "ifa_model_set_tensor_host: global tensor id %d", tensor_id);
     } else {
         IFA_REQUIRE(layer < (int)n->layers.size() && tensor_id >= IFA_LT_NORM1 && tensor_id < IFA_LT_END, "ifa_model_set_tensor_host: layer %d / tensor id %d", layer, tensor_id);
         LLayer &L = n->layers[(size_t)layer];
-        IFA_REQUIRE(expected_shape(n, L.spec, tensor_id, er, ec, vec), "ifa_model_set_tensor_host: tensor %d does not belong to layer %d's mixer", tensor_id, layer);
+        IFA_REQUIRE(expected_shape(n, L.spec, layer, tensor_id, er, ec, vec), "ifa_model_set_tensor_host: tensor %d does not belong to layer %d's mixer", tensor_id, layer);
         t = &L.T(tensor_id);
     }
     const int want = tensor_id == IFA_LT_L_DECAY ? IFA_F32 : IFA_BF16;

@@ -29,12 +29,18 @@ struct LinArgs {
     float alpha; int accumulate, vec;
     int act_c0, act_c1;          // output columns [act_c0, act_c1) pass SiLU after the bias (projections whose consumer wants them activated)
     const bf16_t *norm_w; float norm_eps;      // row kernel, prologue 1: the activations are layer-normed (no bias) on the fly
+    // grouped product (k_lin_mfma only): tile blockIdx.y serves rows [row0, row0 + n) of group g (tile_map {g, row0, n}; *n_tiles valid
+    // tiles) with the matrix W + g * N * K; activation row of output row r: A[a_rows[r]] (a_rows null: r); row_scale per output row
+    const int *tile_map, *n_tiles, *a_rows; const float *row_scale;
+    int act_kind;                              // 1: every output passes the exact (erf) GELU after the bias
 };
 
 __device__ __forceinline__ void lin_store(const LinArgs &P, int t, int n, float acc)
 {
     if (P.bias) acc += bf2f(P.bias[n]);
     if (n >= P.act_c0 && n < P.act_c1) acc = silu_exact(acc);
+    if (P.act_kind == 1) acc = 0.5f * acc * (1.0f + erff(acc * 0.70710678118654752f));
+    if (P.row_scale) acc *= P.row_scale[t];
     if (P.mul) acc *= bf2f(P.mul[n]);
     acc *= P.alpha;
     float *c = P.C + (size_t)t * P.ldc + n;
@@ -52,8 +58,16 @@ __global__ void __launch_bounds__(256) k_lin_mfma(LinArgs P)
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int i = lane & 31, g = lane >> 5;
     const int wm = wave & 1, wn = wave >> 1;
-    const int t0 = blockIdx.y * LM_T, n0 = blockIdx.x * LM_N;
+    int t0 = blockIdx.y * LM_T, t_end = P.T;
+    const int n0 = blockIdx.x * LM_N;
+    const bf16_t *Wg = P.W;
+    if (P.tile_map) {
+        if ((int)blockIdx.y >= *P.n_tiles) return;
+        const int *tm = P.tile_map + 3 * blockIdx.y;
+        Wg += (size_t)tm[0] * P.N * P.K; t0 = tm[1]; t_end = tm[1] + tm[2];
+    }
     const int lr = tid >> 2, lc = (tid & 3) * 8;      // this thread stages 8 consecutive k of row lr
+    const size_t a_row = (t0 + lr < t_end) ? (size_t)(P.a_rows ? P.a_rows[t0 + lr] : t0 + lr) : 0;
     f32x16v acc;
 #pragma unroll
     for (int r = 0; r < 16; r++) acc[r] = 0.0f;
@@ -62,18 +76,18 @@ __global__ void __launch_bounds__(256) k_lin_mfma(LinArgs P)
         float a8[8], w8[8];
         {
             const int t = t0 + lr, n = n0 + lr, k = k0 + lc;
-            const bool in_a = t < P.T, in_w = n < P.N;
+            const bool in_a = t < t_end, in_w = n < P.N;
             if (P.vec && k + 8 <= P.K) {
                 if (in_a) {
-                    const float4 v0 = *reinterpret_cast<const float4 *>(P.A + (size_t)t * P.lda + k);
-                    const float4 v1 = *reinterpret_cast<const float4 *>(P.A + (size_t)t * P.lda + k + 4);
+                    const float4 v0 = *reinterpret_cast<const float4 *>(P.A + a_row * P.lda + k);
+                    const float4 v1 = *reinterpret_cast<const float4 *>(P.A + a_row * P.lda + k + 4);
                     a8[0] = v0.x; a8[1] = v0.y; a8[2] = v0.z; a8[3] = v0.w; a8[4] = v1.x; a8[5] = v1.y; a8[6] = v1.z; a8[7] = v1.w;
                 } else {
 #pragma unroll
                     for (int e = 0; e < 8; e++) a8[e] = 0.0f;
                 }
                 if (in_w) {
-                    const u32x4v wv = *reinterpret_cast<const u32x4v *>(P.W + (size_t)n * P.K + k);
+                    const u32x4v wv = *reinterpret_cast<const u32x4v *>(Wg + (size_t)n * P.K + k);
 #pragma unroll
                     for (int e = 0; e < 4; e++) { w8[2 * e] = __uint_as_float(wv[e] << 16); w8[2 * e + 1] = __uint_as_float(wv[e] & 0xFFFF0000u); }
                 } else {
@@ -84,8 +98,8 @@ __global__ void __launch_bounds__(256) k_lin_mfma(LinArgs P)
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
                     const bool kin = k + e < P.K;
-                    a8[e] = in_a && kin ? P.A[(size_t)t * P.lda + k + e] : 0.0f;
-                    w8[e] = in_w && kin ? bf2f(P.W[(size_t)n * P.K + k + e]) : 0.0f;
+                    a8[e] = in_a && kin ? P.A[a_row * P.lda + k + e] : 0.0f;
+                    w8[e] = in_w && kin ? bf2f(Wg[(size_t)n * P.K + k + e]) : 0.0f;
                 }
             }
         }
@@ -126,7 +140,7 @@ __global__ void __launch_bounds__(256) k_lin_mfma(LinArgs P)
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int t = t0 + 32 * wm + (r & 3) + 8 * (r >> 2) + 4 * g;
-            if (t < P.T) lin_store(P, t, n, acc[r]);
+            if (t < t_end) lin_store(P, t, n, acc[r]);
         }
     }
 }
@@ -223,6 +237,7 @@ static int linear_launch(const void *w_bf16, size_t rows, size_t cols, const voi
     P.T = (int)tokens; P.N = (int)rows; P.K = (int)cols; P.lda = (int)lda; P.ldc = (int)ldc;
     P.alpha = alpha; P.accumulate = accumulate ? 1 : 0; P.act_c0 = silu_col0; P.act_c1 = silu_col1;
     P.norm_w = (const bf16_t *)norm_w_bf16; P.norm_eps = norm_eps;
+    P.tile_map = P.n_tiles = P.a_rows = nullptr; P.row_scale = nullptr; P.act_kind = 0;
     // 16-byte requests need whole 8-element pieces in every row of both operands
     P.vec = (cols % 8 == 0 && lda % 4 == 0 && ((uintptr_t)a_f32 & 15) == 0 && ((uintptr_t)w_bf16 & 15) == 0) ? 1 : 0;
     hipStream_t s = ifa_s(stream);
@@ -262,4 +277,27 @@ extern "C" int ifa_linear_bf16w_rows(int prologue, const void *norm_w_bf16, floa
     IFA_REQUIRE(tokens <= 8, "ifa_linear_bf16w_rows: %zu rows (at most 8)", tokens);
     return linear_launch(w_bf16, rows, cols, a_f32, lda, tokens, bias_bf16, mul_bf16, alpha, accumulate, 1, c_f32, ldc, silu_col0, silu_col1, prologue,
                          norm_w_bf16, norm_eps, stream, "ifa_linear_bf16w_rows");
+}
+
+// Grouped product on the matrix cores: `groups` matrices [rows][cols] back to back in w_bf16; the output rows are sorted by group and
+// cut into tiles of at most 64 rows of ONE group: tile_map_dev[3 i] = {group, first row, rows}, *n_tiles_dev tiles (max_tiles bounds the
+// grid).  C[r][n] = row_scale[r] * act(sum_k A[a_rows[r]][k] W_group[n][k]); a_rows_dev / row_scale_f32 nullable; act 0 none, 1 erf-GELU.
+extern "C" int ifa_linear_bf16w_grouped(const void *w_bf16, size_t rows, size_t cols, int groups, const void *a_f32, size_t lda, const int *a_rows_dev,
+                                        const int *tile_map_dev, const int *n_tiles_dev, size_t max_tiles, const void *row_scale_f32, int act, int ops32,
+                                        void *c_f32, size_t ldc, ifa_stream stream)
+{
+    IFA_REQUIRE(w_bf16 && a_f32 && c_f32 && tile_map_dev && n_tiles_dev, "ifa_linear_bf16w_grouped: null pointer");
+    IFA_REQUIRE(rows > 0 && cols > 0 && groups > 0 && max_tiles > 0 && max_tiles < 65536 && lda >= cols && ldc >= rows && (act == 0 || act == 1), "ifa_linear_bf16w_grouped: bad shape");
+    IFA_REQUIRE(rows < (1u << 30) && cols < (1u << 30), "ifa_linear_bf16w_grouped: dimension too large");
+    LinArgs P;
+    P.W = (const bf16_t *)w_bf16; P.A = (const float *)a_f32; P.C = (float *)c_f32; P.bias = nullptr; P.mul = nullptr;
+    P.T = 0; P.N = (int)rows; P.K = (int)cols; P.lda = (int)lda; P.ldc = (int)ldc; P.alpha = 1.0f; P.accumulate = 0; P.act_c0 = P.act_c1 = 0;
+    P.norm_w = nullptr; P.norm_eps = 0.0f;
+    P.tile_map = tile_map_dev; P.n_tiles = n_tiles_dev; P.a_rows = a_rows_dev; P.row_scale = (const float *)row_scale_f32; P.act_kind = act;
+    P.vec = (cols % 8 == 0 && lda % 4 == 0 && ((uintptr_t)a_f32 & 15) == 0 && ((uintptr_t)w_bf16 & 15) == 0 && (rows * cols) % 8 == 0) ? 1 : 0;
+    const dim3 grid(ifa_cdiv(rows, LM_N), (unsigned)max_tiles);
+    if (ops32) hipLaunchKernelGGL(k_lin_mfma<true>, grid, dim3(256), 0, ifa_s(stream), P);
+    else hipLaunchKernelGGL(k_lin_mfma<false>, grid, dim3(256), 0, ifa_s(stream), P);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
 }

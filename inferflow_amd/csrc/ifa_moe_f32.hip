@@ -1,0 +1,230 @@
+// ifa_moe_f32.hip -- mixture of experts on 32-bit activations with bfloat16 expert matrices:
+//   router   scores = softmax(logits) over `experts` feed-forward experts followed by `identity` identity experts; the `top` largest
+//            (score + correction) are chosen, their weights are the plain scores (not renormalized)
+//   experts  y[t] (+)= sum_k wgt[t][k] * E_{idx[t][k]}(h[t]),  E_e(h) = W_down[e] act(W_up[e] h),  identity: E(h) = h
+// Few rows (decode steps): every (row, choice) pair streams its expert's matrices, a wave per output (k_moe_up_rows / k_moe_down_rows).
+// Many rows: the pairs are sorted by expert (k_moe_sort: counts, offsets and tiles of 64 rows of one expert, all in one workgroup),
+// both products run grouped on the matrix cores (ifa_linear_bf16w_grouped: gather of the rows in the first, activation in its epilogue,
+// the pair's weight in the second's) and k_moe_combine adds a row's pairs in the fixed order of its choices.  No atomics on values: a
+// row's result does not depend on what else is in the step.
+#include <algorithm>
+#include "ifa_host.h"
+#include "ifa_f32_common.h"
+#include "inferflow_amd.h"
+
+using namespace ifa32;
+
+namespace {
+
+typedef uint32_t u32x4m __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float gelu_erf_f(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f)); }
+
+// one wave per row: softmax over n_all logits, then `top` rounds of argmax over score + correction (lowest index on ties)
+__global__ void __launch_bounds__(64) k_moe_route(const float *__restrict__ logits, size_t ld, int n_all, int top, const bf16_t *__restrict__ corr,
+                                                  int *__restrict__ idx, float *__restrict__ wgt)
+{
+    extern __shared__ float sc[];          // [n_all] scores, [n_all] choice scores
+    float *ch = sc + n_all;
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const float *z = logits + (size_t)t * ld;
+    float mx = -INFINITY;
+    for (int e = lane; e < n_all; e += 64) mx = fmaxf(mx, z[e]);
+    mx = wave_max(mx);
+    float sum = 0.0f;
+    for (int e = lane; e < n_all; e += 64) { const float p = expf(z[e] - mx); sc[e] = p; sum += p; }
+    sum = wave_sum(sum);
+    for (int e = lane; e < n_all; e += 64) { const float s = sc[e] / sum; sc[e] = s; ch[e] = s + (corr ? bf2f(corr[e]) : 0.0f); }
+    __syncthreads();
+    for (int k = 0; k < top; k++) {
+        float best = -INFINITY; int bi = 0x7FFFFFFF;
+        for (int e = lane; e < n_all; e += 64) { const float v = ch[e]; if (v > best || (v == best && e < bi)) { best = v; bi = e; } }
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(best, o, 64); const int oi = __shfl_xor(bi, o, 64);
+            if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+        }
+        if (lane == 0) { idx[(size_t)t * top + k] = bi; wgt[(size_t)t * top + k] = sc[bi]; ch[bi] = -INFINITY; }
+        __syncthreads();
+    }
+}
+
+// grid (ff chunks, pairs): act[p][n] = gelu(W_up[e][n] . h[t]); a wave per n at a time.  Identity pairs do nothing.
+__global__ void __launch_bounds__(256) k_moe_up_rows(const float *__restrict__ h, size_t ldh, int W, int F, int experts, int top, const bf16_t *__restrict__ up,
+                                                     const int *__restrict__ idx, float *__restrict__ act, int vec)
+{
+    const int p = blockIdx.y, e = idx[p];
+    if (e >= experts) return;
+    const int lane = threadIdx.x & 63, wave = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6), nwaves = gridDim.x * (blockDim.x >> 6);
+    const float *hr = h + (size_t)(p / top) * ldh;
+    for (int n = wave; n < F; n += nwaves) {
+        const bf16_t *w = up + ((size_t)e * F + n) * W;
+        float acc = 0.0f;
+        if (vec) {
+            for (int k = lane * 8; k < W; k += 512) {
+                const u32x4m wv = *reinterpret_cast<const u32x4m *>(w + k);
+                const float4 a0 = *reinterpret_cast<const float4 *>(hr + k), a1 = *reinterpret_cast<const float4 *>(hr + k + 4);
+                acc = fmaf(a0.x, __uint_as_float(wv[0] << 16), acc); acc = fmaf(a0.y, __uint_as_float(wv[0] & 0xFFFF0000u), acc);
+                acc = fmaf(a0.z, __uint_as_float(wv[1] << 16), acc); acc = fmaf(a0.w, __uint_as_float(wv[1] & 0xFFFF0000u), acc);
+                acc = fmaf(a1.x, __uint_as_float(wv[2] << 16), acc); acc = fmaf(a1.y, __uint_as_float(wv[2] & 0xFFFF0000u), acc);
+                acc = fmaf(a1.z, __uint_as_float(wv[3] << 16), acc); acc = fmaf(a1.w, __uint_as_float(wv[3] & 0xFFFF0000u), acc);
+            }
+        } else {
+            for (int k = lane; k < W; k += 64) acc = fmaf(hr[k], bf2f(w[k]), acc);
+        }
+        acc = wave_sum(acc);
+        if (lane == 0) act[(size_t)p * F + n] = gelu_erf_f(acc);
+    }
+}
+
+// grid (width chunks, rows): y[t][c] (+)= sum_k wgt * (identity ? h[t][c] : W_down[e][c] . act[p]); a wave per c at a time
+__global__ void __launch_bounds__(256) k_moe_down_rows(const float *__restrict__ h, size_t ldh, int W, int F, int experts, int top, const bf16_t *__restrict__ down,
+                                                       const int *__restrict__ idx, const float *__restrict__ wgt, const float *__restrict__ act,
+                                                       int accumulate, float *__restrict__ y, size_t ldy, int vec)
+{
+    const int t = blockIdx.y;
+    const int lane = threadIdx.x & 63, wave = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6), nwaves = gridDim.x * (blockDim.x >> 6);
+    for (int c = wave; c < W; c += nwaves) {
+        float out = 0.0f;
+        for (int k = 0; k < top; k++) {
+            const int p = t * top + k, e = idx[p];
+            const float wk = wgt[p];
+            if (e >= experts) { out = fmaf(wk, h[(size_t)t * ldh + c], out); continue; }
+            const bf16_t *w = down + ((size_t)e * W + c) * F;
+            const float *a = act + (size_t)p * F;
+            float acc = 0.0f;
+            if (vec) {
+                for (int j = lane * 8; j < F; j += 512) {
+                    const u32x4m wv = *reinterpret_cast<const u32x4m *>(w + j);
+                    const float4 a0 = *reinterpret_cast<const float4 *>(a + j), a1 = *reinterpret_cast<const float4 *>(a + j + 4);
+                    acc = fmaf(a0.x, __uint_as_float(wv[0] << 16), acc); acc = fmaf(a0.y, __uint_as_float(wv[0] & 0xFFFF0000u), acc);
+                    acc = fmaf(a0.z, __uint_as_float(wv[1] << 16), acc); acc = fmaf(a0.w, __uint_as_float(wv[1] & 0xFFFF0000u), acc);
+                    acc = fmaf(a1.x, __uint_as_float(wv[2] << 16), acc); acc = fmaf(a1.y, __uint_as_float(wv[2] & 0xFFFF0000u), acc);
+                    acc = fmaf(a1.z, __uint_as_float(wv[3] << 16), acc); acc = fmaf(a1.w, __uint_as_float(wv[3] & 0xFFFF0000u), acc);
+                }
+            } else {
+                for (int j = lane; j < F; j += 64) acc = fmaf(a[j], bf2f(w[j]), acc);
+            }
+            out = fmaf(wk, wave_sum(acc), out);
+        }
+        if (lane == 0) { float *d = y + (size_t)t * ldy + c; *d = accumulate ? *d + out : out; }
+    }
+}
+
+// ONE workgroup: pairs (row, choice) sorted by expert.  a_rows[pos] = row of the pair at sorted place pos, pair_pos[p] = place of pair p
+// (-1: identity), w_sorted[pos] = its weight, tile_map = tiles of at most 64 places of one expert, *n_tiles.  The place of a pair inside
+// its expert's range comes from an LDS counter: the order there may differ from run to run, the values computed per pair do not.
+__global__ void __launch_bounds__(1024) k_moe_sort(const int *__restrict__ idx, const float *__restrict__ wgt, int n_pairs, int experts, int top,
+                                                   int *__restrict__ a_rows, int *__restrict__ pair_pos, float *__restrict__ w_sorted,
+                                                   int *__restrict__ tile_map, int *__restrict__ n_tiles)
+{
+    extern __shared__ int cnt[];           // [experts] counts, then cursors; [experts + 1] offsets
+    int *off = cnt + experts;
+    for (int e = threadIdx.x; e < experts; e += blockDim.x) cnt[e] = 0;
+    __syncthreads();
+    for (int p = threadIdx.x; p < n_pairs; p += blockDim.x) { const int e = idx[p]; if (e < experts) atomicAdd(&cnt[e], 1); }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int o = 0, nt = 0;
+        for (int e = 0; e < experts; e++) {
+            off[e] = o;
+            for (int r = 0; r < cnt[e]; r += 64) { tile_map[3 * nt] = e; tile_map[3 * nt + 1] = o + r; tile_map[3 * nt + 2] = min(64, cnt[e] - r); nt++; }
+            o += cnt[e];
+            cnt[e] = 0;
+        }
+        off[experts] = o;
+        *n_tiles = nt;
+    }
+    __syncthreads();
+    for (int p = threadIdx.x; p < n_pairs; p += blockDim.x) {
+        const int e = idx[p];
+        if (e >= experts) { pair_pos[p] = -1; continue; }
+        const int pos = off[e] + atomicAdd(&cnt[e], 1);
+        a_rows[pos] = p / top; pair_pos[p] = pos; w_sorted[pos] = wgt[p];
+    }
+}
+
+// y[t][c] (+)= sum_k (identity ? wgt h[t][c] : yp[pair_pos][c])  (the pair's weight is already inside yp)
+__global__ void __launch_bounds__(256) k_moe_combine(const float *__restrict__ h, size_t ldh, int W, int top, const int *__restrict__ pair_pos,
+                                                     const float *__restrict__ wgt, const float *__restrict__ yp, int accumulate, float *__restrict__ y, size_t ldy)
+{
+    const int t = blockIdx.y, c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= W) return;
+    float out = 0.0f;
+    for (int k = 0; k < top; k++) {
+        const int p = t * top + k, pos = pair_pos[p];
+        out += pos < 0 ? wgt[p] * h[(size_t)t * ldh + c] : yp[(size_t)pos * W + c];
+    }
+    float *d = y + (size_t)t * ldy + c;
+    *d = accumulate ? *d + out : out;
+}
+
+size_t al16(size_t v) { return (v + 15) & ~(size_t)15; }
+size_t moe_tiles_max(size_t rows, int top, int experts) { return (rows * (size_t)top + 63) / 64 + (size_t)experts; }
+
+} // namespace
+
+extern "C" {
+
+int ifa_moe_route_f32(const void *logits_f32, size_t ld, size_t rows, int n_all, int top, const void *correction_bf16, int *idx_dev, void *wgt_f32,
+                      ifa_stream stream)
+{
+    IFA_REQUIRE(logits_f32 && idx_dev && wgt_f32, "ifa_moe_route_f32: null pointer");
+    IFA_REQUIRE(rows > 0 && n_all >= 1 && n_all <= 4096 && top >= 1 && top <= n_all && ld >= (size_t)n_all, "ifa_moe_route_f32: bad shape (%d router outputs, %d chosen)", n_all, top);
+    hipLaunchKernelGGL(k_moe_route, dim3((unsigned)rows), dim3(64), (size_t)n_all * 8, ifa_s(stream), (const float *)logits_f32, ld, n_all, top,
+                       (const bf16_t *)correction_bf16, idx_dev, (float *)wgt_f32);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+size_t ifa_moe_workspace_bytes(size_t rows, int top, int width, int ff, int experts)
+{
+    const size_t pairs = rows * (size_t)top;
+    return al16(pairs * ff * 4) + al16(pairs * width * 4) + 3 * al16(pairs * 4) + al16(moe_tiles_max(rows, top, experts) * 12) + 16;
+}
+
+int ifa_moe_experts_f32(const void *h_f32, size_t ldh, size_t rows, int width, int ff, int experts, int identity, int top, int act,
+                        const void *up_bf16, const void *down_bf16, const int *idx_dev, const void *wgt_f32, int ops32, void *ws, size_t ws_bytes,
+                        void *y_f32, size_t ldy, int accumulate, ifa_stream stream)
+{
+    IFA_REQUIRE(h_f32 && idx_dev && wgt_f32 && ws && y_f32 && (experts == 0 || (up_bf16 && down_bf16)), "ifa_moe_experts_f32: null pointer");
+    IFA_REQUIRE(rows > 0 && rows < 65536 && width > 0 && ff > 0 && experts >= 0 && experts <= 4096 && identity >= 0 && top >= 1 && top <= experts + identity && act == 0
+                && ldh >= (size_t)width && ldy >= (size_t)width, "ifa_moe_experts_f32: bad shape");
+    IFA_REQUIRE(ws_bytes >= ifa_moe_workspace_bytes(rows, top, width, ff, experts) && ((uintptr_t)ws & 15) == 0, "ifa_moe_experts_f32: workspace of %zu bytes, %zu needed", ws_bytes,
+                ifa_moe_workspace_bytes(rows, top, width, ff, experts));
+    const size_t pairs = rows * (size_t)top;
+    char *b = (char *)ws;
+    float *actb = (float *)b; b += al16(pairs * ff * 4);
+    float *yp = (float *)b; b += al16(pairs * width * 4);
+    int *a_rows = (int *)b; b += al16(pairs * 4);
+    int *pair_pos = (int *)b; b += al16(pairs * 4);
+    float *w_sorted = (float *)b; b += al16(pairs * 4);
+    int *tile_map = (int *)b; b += al16(moe_tiles_max(rows, top, experts) * 12);
+    int *n_tiles = (int *)b;
+    hipStream_t s = ifa_s(stream);
+    const float *h = (const float *)h_f32;
+    if (rows <= 8 || experts == 0) {
+        const int vec_u = (width % 8 == 0 && ldh % 4 == 0 && ((uintptr_t)h_f32 & 15) == 0 && ((uintptr_t)up_bf16 & 15) == 0) ? 1 : 0;
+        const int vec_d = (ff % 8 == 0 && ((uintptr_t)down_bf16 & 15) == 0) ? 1 : 0;
+        if (experts > 0)
+            hipLaunchKernelGGL(k_moe_up_rows, dim3(std::min(64u, ifa_cdiv((size_t)ff, 4)), (unsigned)pairs), dim3(256), 0, s, h, ldh, width, ff, experts, top,
+                               (const bf16_t *)up_bf16, idx_dev, actb, vec_u);
+        hipLaunchKernelGGL(k_moe_down_rows, dim3(std::min(256u, ifa_cdiv((size_t)width, 4)), (unsigned)rows), dim3(256), 0, s, h, ldh, width, ff, experts, top,
+                           (const bf16_t *)down_bf16, idx_dev, (const float *)wgt_f32, actb, accumulate ? 1 : 0, (float *)y_f32, ldy, vec_d);
+        IFA_LAUNCH_CHECK();
+        return IFA_OK;
+    }
+    const size_t max_tiles = moe_tiles_max(rows, top, experts);
+    IFA_REQUIRE(max_tiles < 65536, "ifa_moe_experts_f32: %zu rows x %d choices exceed one step", rows, top);
+    hipLaunchKernelGGL(k_moe_sort, dim3(1), dim3(1024), (size_t)(2 * experts + 1) * 4, s, idx_dev, (const float *)wgt_f32, (int)pairs, experts, top, a_rows, pair_pos, w_sorted,
+                       tile_map, n_tiles);
+    IFA_LAUNCH_CHECK();
+    int rc;
+    if ((rc = ifa_linear_bf16w_grouped(up_bf16, (size_t)ff, (size_t)width, experts, h_f32, ldh, a_rows, tile_map, n_tiles, max_tiles, nullptr, 1, ops32, actb, (size_t)ff, stream))) return rc;
+    if ((rc = ifa_linear_bf16w_grouped(down_bf16, (size_t)width, (size_t)ff, experts, actb, (size_t)ff, nullptr, tile_map, n_tiles, max_tiles, w_sorted, 0, ops32, yp, (size_t)width, stream))) return rc;
+    hipLaunchKernelGGL(k_moe_combine, dim3(ifa_cdiv((size_t)width, 256), (unsigned)rows), dim3(256), 0, s, h, ldh, width, top, pair_pos, (const float *)wgt_f32, yp,
+                       accumulate ? 1 : 0, (float *)y_f32, ldy);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+} // extern "C"

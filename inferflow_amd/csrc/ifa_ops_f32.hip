@@ -46,6 +46,53 @@ __global__ void __launch_bounds__(256) k_norm_f32(int kind, const float *__restr
     }
 }
 
+// x[t][c] = embed[token_t][c], no position vector
+__global__ void __launch_bounds__(256) k_embed_rows(const bf16_t *__restrict__ embed, int vocab, int width, const int *__restrict__ tokens, float *__restrict__ x)
+{
+    const int t = blockIdx.x;
+    const int tok = min(max(tokens[t], 0), vocab - 1);
+    for (int c = threadIdx.x; c < width; c += blockDim.x) x[(size_t)t * width + c] = bf2f(embed[(size_t)tok * width + c]);
+}
+
+// RMS norm in `groups` consecutive parts of a row, a wave per part at a time: y (+)= x / sqrt(mean_part(x^2) + eps) * w
+__global__ void __launch_bounds__(256) k_group_rmsnorm(const float *__restrict__ x, size_t ldx, int cols, int groups, const bf16_t *__restrict__ w, float eps,
+                                                       int accumulate, float *__restrict__ y, size_t ldy)
+{
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const float *xr = x + (size_t)blockIdx.x * ldx;
+    float *yr = y + (size_t)blockIdx.x * ldy;
+    const int gs = cols / groups;
+    for (int g = wave; g < groups; g += nw) {
+        float q = 0.0f;
+        for (int c = lane; c < gs; c += 64) { const float v = xr[g * gs + c]; q = fmaf(v, v, q); }
+        const float rinv = 1.0f / sqrtf(wave_sum(q) / (float)gs + eps);
+        for (int c = lane; c < gs; c += 64) {
+            const int cc = g * gs + c;
+            float v = xr[cc] * rinv;
+            if (w) v *= bf2f(w[cc]);
+            yr[cc] = accumulate ? yr[cc] + v : v;
+        }
+    }
+}
+
+// stack[count - 1] <- x; x <- sum_j w[j] stack[j]  (element-wise over n = rows * cols values)
+__global__ void __launch_bounds__(256) k_depth_average(float *__restrict__ x, size_t n, float *__restrict__ stack, size_t plane, int count, const bf16_t *__restrict__ w)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    const float cur = x[i];
+    stack[(size_t)(count - 1) * plane + i] = cur;
+    float s = 0.0f;
+    for (int j = 0; j + 1 < count; j++) s = fmaf(bf2f(w[j]), stack[(size_t)j * plane + i], s);
+    x[i] = fmaf(bf2f(w[count - 1]), cur, s);
+}
+
+__global__ void __launch_bounds__(256) k_softcap(float *__restrict__ x, size_t n, float cap)
+{
+    const size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) x[i] = cap * tanhf(x[i] / cap);
+}
+
 // out[t][c] = act(gu[t][c]) * gu[t][F + c]
 __global__ void __launch_bounds__(256) k_glu_f32(int kind, const float *__restrict__ gu, size_t ld, int F, float *__restrict__ out, size_t ldo)
 {
@@ -99,6 +146,45 @@ int ifa_embed_sinpos_f32(const void *embed_bf16, int vocab, int width, const int
     IFA_REQUIRE(vocab > 0 && width > 0 && tokens > 0 && base > 1.0f, "ifa_embed_sinpos_f32: bad shape");
     hipLaunchKernelGGL(k_embed_sinpos, dim3((unsigned)tokens), dim3(256), 0, ifa_s(stream), (const bf16_t *)embed_bf16, vocab, width, tokens_dev,
                        positions_dev, log((double)base), (float *)x_f32);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_embed_rows_f32(const void *embed_bf16, int vocab, int width, const int *tokens_dev, size_t tokens, void *x_f32, ifa_stream stream)
+{
+    IFA_REQUIRE(embed_bf16 && tokens_dev && x_f32, "ifa_embed_rows_f32: null pointer");
+    IFA_REQUIRE(vocab > 0 && width > 0 && tokens > 0, "ifa_embed_rows_f32: bad shape");
+    hipLaunchKernelGGL(k_embed_rows, dim3((unsigned)tokens), dim3(256), 0, ifa_s(stream), (const bf16_t *)embed_bf16, vocab, width, tokens_dev, (float *)x_f32);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_group_rmsnorm_f32(const void *x_f32, size_t ldx, size_t rows, size_t cols, int groups, const void *w_bf16, float eps, int accumulate,
+                          void *y_f32, size_t ldy, ifa_stream stream)
+{
+    IFA_REQUIRE(x_f32 && y_f32, "ifa_group_rmsnorm_f32: null pointer");
+    IFA_REQUIRE(rows > 0 && cols > 0 && groups >= 1 && cols % (size_t)groups == 0 && ldx >= cols && ldy >= cols, "ifa_group_rmsnorm_f32: bad arguments (%zu columns in %d parts)", cols, groups);
+    IFA_REQUIRE(!accumulate || x_f32 != y_f32, "ifa_group_rmsnorm_f32: accumulating a row's norm into the row itself");
+    hipLaunchKernelGGL(k_group_rmsnorm, dim3((unsigned)rows), dim3(256), 0, ifa_s(stream), (const float *)x_f32, ldx, (int)cols, groups, (const bf16_t *)w_bf16, eps,
+                       accumulate ? 1 : 0, (float *)y_f32, ldy);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_depth_average_f32(void *x_f32, size_t rows, size_t cols, void *stack_f32, size_t plane_stride, int count, const void *w_bf16, ifa_stream stream)
+{
+    IFA_REQUIRE(x_f32 && stack_f32 && w_bf16, "ifa_depth_average_f32: null pointer");
+    IFA_REQUIRE(rows > 0 && cols > 0 && count >= 1 && plane_stride >= rows * cols, "ifa_depth_average_f32: bad arguments");
+    const size_t n = rows * cols;
+    hipLaunchKernelGGL(k_depth_average, dim3(ifa_cdiv(n, 256)), dim3(256), 0, ifa_s(stream), (float *)x_f32, n, (float *)stack_f32, plane_stride, count, (const bf16_t *)w_bf16);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_softcap_f32(void *x_f32, size_t n, float cap, ifa_stream stream)
+{
+    IFA_REQUIRE(x_f32 && n > 0 && cap > 0.0f, "ifa_softcap_f32: bad arguments");
+    hipLaunchKernelGGL(k_softcap, dim3(ifa_cdiv(n, 256)), dim3(256), 0, ifa_s(stream), (float *)x_f32, n, cap);
     IFA_LAUNCH_CHECK();
     return IFA_OK;
 }

@@ -57,6 +57,28 @@ __global__ void __launch_bounds__(256) k_shortconv_silu(const float *__restrict_
     for (int c = c_lo + threadIdx.x; c < c_hi; c += blockDim.x) y[(size_t)t * ldy + c] = c < scale_cols ? ys[c - c_lo] * qscale : ys[c - c_lo];
 }
 
+// y[t][c] = x[t][c] + sum_j w[c][j] * x_(t - taps + 1 + j)[c]: the same causal taps without activation, added to the input itself
+__global__ void __launch_bounds__(256) k_shortconv_residual(const float *__restrict__ x, size_t ldx, int C, int taps, const bf16_t *__restrict__ w,
+                                                            const SeqDesc *__restrict__ seqs, const int *__restrict__ row_seq,
+                                                            float *const *__restrict__ slot_base, size_t state_off, float *__restrict__ y, size_t ldy)
+{
+    const int t = blockIdx.x;
+    const SeqDesc sd = seqs[row_seq[t]];
+    const int i = t - sd.row0;
+    const float *tail = sd.pos0 > 0 ? slot_base[sd.slot] + state_off : nullptr;
+    for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < C; c += gridDim.y * blockDim.x) {
+        float acc = 0.0f;
+        for (int j = 0; j < taps; j++) {
+            const int idx = i - (taps - 1) + j;
+            float v;
+            if (idx >= 0) v = x[(size_t)(sd.row0 + idx) * ldx + c];
+            else v = tail ? tail[(size_t)(taps - 1 + idx) * C + c] : 0.0f;
+            acc = fmaf(bf2f(w[(size_t)c * taps + j]), v, acc);
+        }
+        y[(size_t)t * ldy + c] = x[(size_t)t * ldx + c] + acc;
+    }
+}
+
 // grid: one workgroup per sequence.  The carried tail becomes the last taps - 1 inputs of (old tail, this step's rows).
 __global__ void __launch_bounds__(256) k_shortconv_tail(const float *__restrict__ x, size_t ldx, int C, int taps, const SeqDesc *__restrict__ seqs,
                                                         float *const *__restrict__ slot_base, size_t state_off)
@@ -332,6 +354,17 @@ int ifa_shortconv_silu_f32(const void *x_f32, size_t ldx, int channels, int taps
     hipLaunchKernelGGL(k_shortconv_silu, dim3((unsigned)rows, ifa_cdiv((size_t)channels, (size_t)slice)), dim3(256), (size_t)slice * 4, ifa_s(stream),
                        (const float *)x_f32, ldx, channels, taps, (const bf16_t *)w_bf16, (const SeqDesc *)seqs_dev, row_seq_dev, (float *const *)slot_base_dev,
                        state_off, norm_cols, group_dim, l2_eps, scale_cols, scale, (float *)y_f32, ldy, slice);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_shortconv_residual_f32(const void *x_f32, size_t ldx, int channels, int taps, const void *w_bf16, const void *seqs_dev, const int *row_seq_dev,
+                               size_t rows, void *const *slot_base_dev, size_t state_off, void *y_f32, size_t ldy, ifa_stream stream)
+{
+    IFA_REQUIRE(x_f32 && w_bf16 && seqs_dev && row_seq_dev && slot_base_dev && y_f32 && x_f32 != y_f32, "ifa_shortconv_residual_f32: null pointer or y = x");
+    IFA_REQUIRE(channels > 0 && taps >= 1 && taps <= 64 && rows > 0 && ldx >= (size_t)channels && ldy >= (size_t)channels, "ifa_shortconv_residual_f32: bad shape");
+    hipLaunchKernelGGL(k_shortconv_residual, dim3((unsigned)rows, std::min(8u, ifa_cdiv((size_t)channels, 256))), dim3(256), 0, ifa_s(stream), (const float *)x_f32, ldx,
+                       channels, taps, (const bf16_t *)w_bf16, (const SeqDesc *)seqs_dev, row_seq_dev, (float *const *)slot_base_dev, state_off, (float *)y_f32, ldy);
     IFA_LAUNCH_CHECK();
     return IFA_OK;
 }

@@ -7,6 +7,14 @@
 //   "parallel"  windowed softmax attention with kept first tokens, soft cap, distance-bucket bias and sink ("left") beside
 //               decayed linear attention ("right"), summed with left_scale / right_scale
 //   "delta"     gated delta rule behind short causal convolutions
+//
+// Muzopel: width / vocab / norm.eps / norm.groups / canon.taps / logit_softcap; the embedding and the output pass a grouped RMS norm;
+// every layer reads the residual through a short causal convolution, puts a grouped RMS norm on each sub-layer's output, feeds
+// forward through a mixture of experts (with identity experts and a correction on the choice scores) and ends in a learned average
+// over the depth of the stack; mixer types
+//   "latent_attention"    queries through a normed latent (q_rank), YaRN-scaled rotation when rot.scaling is given, sigmoid gate per head
+//   "latent_attention_2"  queries straight from the input, plain rotation, no gate
+// both with one cached row [kv_rank latent | rot_dim rotated key part] per position.
 #include <cmath>
 #include <cstdio>
 #include <cstring>
@@ -97,6 +105,89 @@ bool ParseGelarax(const JsonValue &root, LayeredDesc &d)
     return true;
 }
 
+// ---- Muzopel
+bool ParseMuzopel(const JsonValue &root, LayeredDesc &d)
+{
+    memset(&d.cfg, 0, sizeof(d.cfg));
+    if (!Need(root, "width", d.cfg.width, "config") || !Need(root, "vocab", d.cfg.vocab, "config")) return false;
+    const JsonValue *norm = root.Get("norm");
+    if (!norm) { EngineSetError("config.json: norm is missing"); return false; }
+    if (!Need(*norm, "eps", d.cfg.eps, "norm") || !Need(*norm, "groups", d.cfg.norm_groups, "norm")) return false;
+    d.cfg.stem = 1;
+    root.GetNumber("logit_softcap", d.cfg.logit_softcap);
+    int taps = 0;
+    if (const JsonValue *canon = root.Get("canon")) canon->GetNumber("taps", taps);
+    const JsonValue *layers = root.Get("layers");
+    if (!layers || layers->type != JsonValue::Array || layers->arr.empty()) { EngineSetError("config.json: layers is missing or empty"); return false; }
+    for (size_t li = 0; li < layers->arr.size(); li++) {
+        const JsonValue &L = layers->arr[li];
+        ifa_layer_spec s; memset(&s, 0, sizeof(s));
+        std::string type;
+        const JsonValue *mx = L.Get("mixer");
+        if (!L.GetString("type", type) || !mx || mx->type != JsonValue::Object) { EngineSetError("config.json: layer %zu has no type / mixer", li); return false; }
+        if (type != "latent_attention" && type != "latent_attention_2") { EngineSetError("config.json: layer %zu: unknown type \"%s\"", li, type.c_str()); return false; }
+        const bool first = type == "latent_attention";
+        s.mixer = IFA_MIX_LATENT; s.block = IFA_BLOCK_POSTNORM; s.canon_taps = taps; s.depth_avg = 1;
+        if (!Need(*mx, "heads", s.m_heads, "mixer") || !Need(*mx, "dim", s.m_dim, "mixer") || !Need(*mx, "rot_dim", s.m_rot_dim, "mixer") || !Need(*mx, "vdim", s.m_vdim, "mixer")
+            || !Need(*mx, "kv_rank", s.m_kv_rank, "mixer") || !Need(*mx, "scale", s.m_scale, "mixer")) return false;
+        if (first && !Need(*mx, "q_rank", s.m_q_rank, "mixer")) return false;
+        s.m_gate = first ? 1 : 0;
+        const JsonValue *rot = mx->Get("rot");
+        if (!rot || !Need(*rot, "base", s.m_rot_base, "mixer.rot") || !Need(*rot, "dims", s.m_rot_dims, "mixer.rot")) { if (!rot) EngineSetError("config.json: layer %zu: mixer.rot is missing", li); return false; }
+        const JsonValue *sc = rot->Get("scaling");
+        if (first && sc && sc->type == JsonValue::Object
+            && (!Need(*sc, "factor", s.m_yarn_factor, "rot.scaling") || !Need(*sc, "original", s.m_yarn_original, "rot.scaling")
+                || !Need(*sc, "fast", s.m_yarn_fast, "rot.scaling") || !Need(*sc, "slow", s.m_yarn_slow, "rot.scaling"))) return false;
+        const JsonValue *mlp = L.Get("mlp");
+        if (mlp && mlp->type == JsonValue::Object) {
+            std::string kind;
+            if (!mlp->GetString("kind", kind) || kind != "moe") { EngineSetError("config.json: layer %zu: mlp.kind \"%s\" is not supported (moe)", li, kind.c_str()); return false; }
+            const JsonValue *ex = mlp->Get("expert"), *ro = mlp->Get("router");
+            if (!ex || !ro) { EngineSetError("config.json: layer %zu: mlp needs expert and router", li); return false; }
+            s.ffn_kind = IFA_FFN_MOE;
+            if (!Need(*ex, "ff", s.x_ff, "mlp.expert") || !Need(*ro, "experts", s.x_experts, "mlp.router") || !Need(*ro, "top", s.x_top, "mlp.router")) return false;
+            ro->GetNumber("identity", s.x_identity);
+        }
+        d.layers.push_back(s);
+        d.decays.push_back(std::vector<float>());
+    }
+    d.cfg.n_layers = (int)d.layers.size();
+    return true;
+}
+
+// tensor name -> (layer, id).  Names that share (layer, id) are parts of ONE tensor, stacked row-wise in the order given (the experts).
+void MuzopelNames(const LayeredDesc &d, std::vector<std::pair<std::string, std::pair<int, int>>> &out)
+{
+    out.push_back({"embed", {-1, IFA_T_EMBD}});
+    out.push_back({"embed.norm", {-1, IFA_T_EMBD_NORM}});
+    out.push_back({"final.norm", {-1, IFA_T_OUT_NORM}});
+    out.push_back({"head", {-1, IFA_T_LM_HEAD}});
+    for (size_t li = 0; li < d.layers.size(); li++) {
+        const ifa_layer_spec &s = d.layers[li];
+        const std::string p = "l" + std::to_string(li) + ".";
+        const int l = (int)li;
+        const bool moe = s.ffn_kind == IFA_FFN_MOE && s.x_experts + s.x_identity > 0;
+        out.push_back({p + "norm1", {l, IFA_LT_NORM1}});
+        if (s.canon_taps > 0) out.push_back({p + "canon1", {l, IFA_LT_CANON1}});
+        out.push_back({p + "dwa", {l, IFA_LT_DWA}});
+        if (s.m_q_rank > 0) {
+            out.push_back({p + "mix.dq", {l, IFA_LT_M_DQ}}); out.push_back({p + "mix.dq.norm", {l, IFA_LT_M_DQ_NORM}}); out.push_back({p + "mix.uq", {l, IFA_LT_M_UQ}});
+        } else out.push_back({p + "mix.q", {l, IFA_LT_M_Q}});
+        out.push_back({p + "mix.dkv", {l, IFA_LT_M_DKV}}); out.push_back({p + "mix.dkv.norm", {l, IFA_LT_M_DKV_NORM}});
+        out.push_back({p + "mix.uk", {l, IFA_LT_M_UK}}); out.push_back({p + "mix.uv", {l, IFA_LT_M_UV}});
+        if (s.m_gate) out.push_back({p + "mix.g", {l, IFA_LT_M_G}});
+        out.push_back({p + "mix.o", {l, IFA_LT_M_O}});
+        if (!moe) continue;
+        out.push_back({p + "norm2", {l, IFA_LT_NORM2}});
+        if (s.canon_taps > 0) out.push_back({p + "canon2", {l, IFA_LT_CANON2}});
+        out.push_back({p + "mlp.router", {l, IFA_LT_X_ROUTER}}); out.push_back({p + "mlp.correction", {l, IFA_LT_X_CORR}});
+        for (int e = 0; e < s.x_experts; e++) out.push_back({p + "mlp.e" + std::to_string(e) + ".up", {l, IFA_LT_X_UP}});
+        for (int e = 0; e < s.x_experts; e++) out.push_back({p + "mlp.e" + std::to_string(e) + ".down", {l, IFA_LT_X_DOWN}});
+    }
+}
+
+bool NoSizesFromTensors(const std::map<std::string, StTensorEntry> &, LayeredDesc &) { return true; }
+
 struct NameId { const char *suffix; int id; };
 const NameId kGelaraxCommon[] = {{"norm1", IFA_LT_NORM1}, {"ls1", IFA_LT_LS1}, {"ls2", IFA_LT_LS2}, {"mlp.gate", IFA_LT_FFN_GATE}, {"mlp.gate.b", IFA_LT_FFN_GATE_B},
                                  {"mlp.up", IFA_LT_FFN_UP}, {"mlp.up.b", IFA_LT_FFN_UP_B}, {"mlp.down", IFA_LT_FFN_DOWN}, {"mlp.down.b", IFA_LT_FFN_DOWN_B}};
@@ -144,7 +235,8 @@ struct ArchEntry {
     bool (*sizes_from_tensors)(const std::map<std::string, StTensorEntry> &index, LayeredDesc &d);
     void (*names)(const LayeredDesc &d, std::vector<std::pair<std::string, std::pair<int, int>>> &out);
 };
-const ArchEntry kArchitectures[] = {{"Gelarax", ParseGelarax, GelaraxSizesFromTensors, GelaraxNames}};
+const ArchEntry kArchitectures[] = {{"Gelarax", ParseGelarax, GelaraxSizesFromTensors, GelaraxNames},
+                                    {"Muzopel", ParseMuzopel, NoSizesFromTensors, MuzopelNames}};
 
 const ArchEntry *FindArch(const std::string &name)
 {
@@ -207,8 +299,10 @@ bool LoadLayered(std::vector<WorkerPlan> &plans, ModelSpec &spec)
     if (ifa_model_create_layered(&d.cfg, d.layers.data(), &w.model) != IFA_OK) { EngineSetError("ifa_model_create_layered: %s", ifa_last_error()); return false; }
     std::vector<std::pair<std::string, std::pair<int, int>>> names;
     arch->names(d, names);
-    std::vector<uint8_t> raw;
-    for (const auto &nm : names) {
+    std::vector<uint8_t> raw, stacked;
+    size_t stacked_rows = 0, stacked_cols = 0;
+    for (size_t ni = 0; ni < names.size(); ni++) {
+        const auto &nm = names[ni];
         auto it = index.find(nm.first);
         if (it == index.end()) { EngineSetError("tensor %s is missing in %s", nm.first.c_str(), spec.dir.c_str()); return false; }
         const StTensorEntry &e = it->second;
@@ -222,10 +316,19 @@ bool LoadLayered(std::vector<WorkerPlan> &plans, ModelSpec &spec)
         const bool ok = fread(raw.data(), 1, raw.size(), fp) == raw.size();
         fclose(fp);
         if (!ok) { EngineSetError("%s is truncated (tensor %s)", e.file.c_str(), nm.first.c_str()); return false; }
-        const size_t rows = e.shape.size() >= 2 ? e.shape[0] : 1, cols = e.shape.size() >= 2 ? cnt / e.shape[0] : cnt;
-        if (ifa_model_set_tensor_host(w.model, nm.second.first, nm.second.second, IFA_BF16, raw.data(), rows, cols) != IFA_OK) {
-            EngineSetError("tensor %s: %s", nm.first.c_str(), ifa_last_error()); return false;
+        size_t rows = e.shape.size() >= 2 ? e.shape[0] : 1, cols = e.shape.size() >= 2 ? cnt / e.shape[0] : cnt;
+        // consecutive names with the same (layer, id) are parts of one tensor, stacked row-wise
+        const bool more = ni + 1 < names.size() && names[ni + 1].second == nm.second, part = more || !stacked.empty();
+        if (part) {
+            if (!stacked.empty() && cols != stacked_cols) { EngineSetError("tensor %s: %zu columns, the parts before it have %zu", nm.first.c_str(), cols, stacked_cols); return false; }
+            stacked.insert(stacked.end(), raw.begin(), raw.end());
+            stacked_rows += rows; stacked_cols = cols;
+            if (more) continue;
+            rows = stacked_rows;
         }
+        const int rc = ifa_model_set_tensor_host(w.model, nm.second.first, nm.second.second, IFA_BF16, part ? stacked.data() : raw.data(), rows, cols);
+        stacked.clear(); stacked_rows = 0;
+        if (rc != IFA_OK) { EngineSetError("tensor %s: %s", nm.first.c_str(), ifa_last_error()); return false; }
     }
     for (size_t li = 0; li < d.layers.size(); li++)
         if (d.layers[li].mixer == IFA_MIX_WINDOW_LINEAR
