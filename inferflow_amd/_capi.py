@@ -162,6 +162,20 @@ SIGNATURES = {
     "ifa_gated_groupnorm_f32": (_i, [_vp, _sz, _sz, _i, _i, _vp, _i, _vp, _sz, _i, _f, _vp, _sz, _vp]),
     "ifa_kv_store_f32": (_i, [_vp, _sz, _vp, _sz, _i, _i, _i, _f, _vp, _vp, _sz, _vp, _sz, _sz, _vp]),
     "ifa_attention_window_f32": (_i, [_vp, _sz, _i, _i, _i, _i, _f, _f, _f, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _sz, _vp, _sz, _sz, _vp, _sz, _vp, _i, _i, _vp, _sz, _vp]),
+    "ifa_linear_bf16w_grouped": (_i, [_vp, _sz, _sz, _i, _vp, _sz, _vp, _vp, _vp, _sz, _vp, _i, _i, _vp, _sz, _vp]),
+    "ifa_embed_rows_f32": (_i, [_vp, _i, _i, _vp, _sz, _vp, _vp]),
+    "ifa_group_rmsnorm_f32": (_i, [_vp, _sz, _sz, _sz, _i, _vp, _f, _i, _vp, _sz, _vp]),
+    "ifa_shortconv_residual_f32": (_i, [_vp, _sz, _i, _i, _vp, _vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp]),
+    "ifa_depth_average_f32": (_i, [_vp, _sz, _sz, _vp, _sz, _i, _vp, _vp]),
+    "ifa_softcap_f32": (_i, [_vp, _sz, _f, _vp]),
+    "ifa_latent_prepare_f32": (_i, [_vp, _sz, _i, _i, _i, _vp, _f, _vp, _sz, _i, _i, _vp, _f, _vp, _vp, _sz, _vp, _sz, _vp]),
+    "ifa_latent_absorb_q_f32": (_i, [_vp, _sz, _i, _i, _i, _i, _vp, _sz, _vp, _sz, _vp]),
+    "ifa_latent_expand_out_f32": (_i, [_vp, _sz, _i, _i, _i, _i, _vp, _vp, _sz, _sz, _vp, _sz, _vp]),
+    "ifa_attention_latent_tile_f32": (_i, [_vp, _sz, _i, _i, _i, _i, _i, _f, _vp, _sz, _vp, _sz, _vp, _vp, _sz, _vp, _vp, _i, _vp, _sz, _vp, _sz, _vp]),
+    "ifa_attention_latent_tile_fits": (_i, [_i, _i, _i]),
+    "ifa_moe_route_f32": (_i, [_vp, _sz, _sz, _i, _i, _vp, _vp, _vp, _vp]),
+    "ifa_moe_workspace_bytes": (_sz, [_sz, _i, _i, _i, _i]),
+    "ifa_moe_experts_f32": (_i, [_vp, _sz, _sz, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _sz, _vp, _sz, _i, _vp]),
     "ifa_model_create_layered": (_i, [_vp, _vp, C.POINTER(_vp)]),
     "ifa_model_set_tensor_host": (_i, [_vp, _i, _i, _i, _vp, _sz, _sz]),
     "ifa_model_logits_f32": (_i, [_vp, C.POINTER(_vp), C.POINTER(_sz), C.POINTER(_sz)]),
