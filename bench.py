@@ -376,7 +376,90 @@ ARCH_SIZES = {      # --arch gelarax: layer sizes that resemble a real model's, 
 }
 
 
+MUZOPEL_SIZES = {   # --arch muzopel: eight layers each (three latent-attention layers with direct queries, one with latent queries, twice), a mixture of experts in every layer
+    "w1024": dict(width=1024, heads=8, dim=96, rot_dim=32, vdim=128, kv_rank=256, q_rank=384, experts=16, identity=2, top=4, ff=704),
+    "w2048": dict(width=2048, heads=16, dim=128, rot_dim=64, vdim=128, kv_rank=512, q_rank=768, experts=32, identity=2, top=6, ff=1408),
+}
+
+
 def run_arch_bench(args):
+    """--arch gelarax | muzopel: see run_gelarax_bench / the Muzopel branch below"""
+    if args.arch.lower() == "muzopel":
+        return run_muzopel_bench(args)
+    return run_gelarax_bench(args)
+
+
+def run_muzopel_bench(args):
+    """--arch muzopel: prefill and decode throughput of Muzopel-shaped models with random bfloat16 weights (layer-list worker: latent attention, mixture
+    of experts, fp32 residual) beside the closest standard model of this framework at equal width / heads / layers / experts / expert width (Mixtral
+    wiring: full-head attention with an F16 KV cache, gated experts, F16 weights).  One JSON line; `value` = decode tokens/s of the largest size."""
+    import shutil
+    import tempfile
+    import numpy as np
+    import torch
+    from inferflow_amd import dtypes as dt, synth
+    from inferflow_amd.engine import InferenceEngine
+    torch.cuda.set_device(0)
+    lens = [int(x) for x in args.prefill_lens.split(",") if x]
+    steps, warmup = args.steps, args.warmup
+    sizes = [x for x in args.arch_sizes.split(",") if x]
+    ctx = max(lens) + warmup + steps + 8
+    rng = np.random.default_rng(42)
+    rows = []
+
+    def timed(fn):
+        torch.cuda.synchronize(); t0 = time.perf_counter(); fn(); torch.cuda.synchronize()
+        return time.perf_counter() - t0
+
+    for name in sizes:
+        sz = MUZOPEL_SIZES[name]
+        cfg = synth.muzopel_config(vocab=32000, **sz)
+        d = tempfile.mkdtemp(prefix="ifa_muzopel_", dir="/dev/shm" if os.path.isdir("/dev/shm") else None)
+        try:
+            synth.write_muzopel_dir(d, cfg, seed=1)
+            eng = InferenceEngine.from_model_dir(d, "bfloat16", ctx, 2, False)
+        finally:
+            shutil.rmtree(d, ignore_errors=True)
+        shapes = synth.muzopel_tensor_shapes(cfg)
+        g = {"prefill_tok_s": {}, "params": int(sum(int(np.prod(s)) for s in shapes.values()))}
+        for n in lens:
+            prompt = [int(t) for t in rng.integers(3, 32000, n)]
+            best = 1e9
+            for rep in range(3):
+                q = eng.add_query(prompt)
+                best = min(best, timed(lambda: eng.generate(q, 1)))
+                if rep < 2:
+                    eng.remove_query(q)
+            g["prefill_tok_s"][str(n)] = n / best
+        if warmup > 0:
+            eng.generate(q, warmup)
+        wall = timed(lambda: eng.generate(q, steps))
+        g["decode_tok_s"] = steps / wall; g["decode_ms_per_step"] = wall * 1e3 / steps; g["decode_context"] = "%d..%d" % (lens[-1] + warmup, lens[-1] + warmup + steps)
+        eng.close()
+        # the closest standard model: same width, heads, layer count, experts, choices per token and expert width, F16 weights
+        synth.SHAPES["cmp_" + name] = dict(dim=sz["width"], layers=8, heads=sz["heads"], kv_heads=sz["heads"], head_dim=128, ffn=sz["ff"], vocab=32000,
+                                           experts=sz["experts"], moe_top_k=sz["top"])
+        wk, _, _ = synth.build("cmp_" + name, dt.F16, dt.F16, ctx, quant_threshold=1 << 62)
+        c = {"prefill_tok_s": {}}
+        for n in lens:
+            prompt = rng.integers(3, 32000, n).astype(np.int32)
+            best = min(timed(lambda: wk.forward(prompt, 0)) for _ in range(3))
+            c["prefill_tok_s"][str(n)] = n / best
+        nxt = int(wk.forward(prompt, 0))
+        if warmup > 0:
+            wk.decode(nxt, lens[-1], warmup)
+        wall = timed(lambda: wk.decode(nxt, lens[-1] + warmup, steps))
+        c["decode_tok_s"] = steps / wall; c["decode_ms_per_step"] = wall * 1e3 / steps
+        del wk
+        rows.append({"size": name, "layers": 8, **sz, "muzopel": g, "closest_standard_model": c})
+    last = rows[-1]["muzopel"]
+    print(json.dumps({"metric": "decode tokens/sec, Muzopel-shaped model (%s), batch=1 greedy" % sizes[-1], "value": last["decode_tok_s"], "unit": "tokens/s", "n_gpus": 1,
+                      "steps": steps, "warmup": warmup, "ms_per_step": last["decode_ms_per_step"], "higher_is_better": True, "scaling": "strong", "vs_baseline": None,
+                      "dtype": "bf16 weights and matrix-product operands, f32 accumulation, residual, scores and cache", "data": "synthetic",
+                      "config": {"model": "Muzopel-shaped, random weights", "global_batch": 1, "seq_len": lens[-1], "parallelism": "single"}, "sizes": rows}))
+
+
+def run_gelarax_bench(args):
     """--arch gelarax: prefill and decode throughput of Gelarax-shaped models with random bfloat16 weights (layer-list worker, fp32 residual) beside
     the closest standard model of this framework at equal width / FFN / heads / layers (Llama wiring, F16 weights, F16 KV cache, same kernels as the
     headline path with the quantiser switched off).  One JSON line; `value` = decode tokens/s of the largest Gelarax size."""
@@ -465,13 +548,13 @@ def main():
                     "a functional check of the N > 1 step logic on a one-GPU box, not a scaling number")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--cpu-tokens", type=int, default=0, help="CPU baseline sample size (0 = auto)")
-    ap.add_argument("--arch", default="", help="'gelarax': instead of the headline workload, prefill / decode rates of Gelarax-shaped models beside the "
+    ap.add_argument("--arch", default="", help="'gelarax' or 'muzopel': instead of the headline workload, prefill / decode rates of models of that design beside the "
                     "closest standard model at equal size (one GPU; --prefill-lens, --steps, --warmup apply)")
     ap.add_argument("--arch-sizes", default="w1024,w2048")
     args = ap.parse_args()
     if args.arch:
-        if args.arch.lower() != "gelarax":
-            raise SystemExit("unknown --arch %s (gelarax)" % args.arch)
+        if args.arch.lower() not in ("gelarax", "muzopel"):
+            raise SystemExit("unknown --arch %s (gelarax, muzopel)" % args.arch)
         if args.gpus > 1 or int(os.environ.get("WORLD_SIZE", "1")) > 1:
             raise SystemExit("--arch runs on one GPU")
         return run_arch_bench(args)

@@ -168,7 +168,52 @@ def gelarax_tensor_shapes(cfg, buckets=32):
     return s
 
 
-def write_gelarax_dir(path, cfg, seed=0):
+def muzopel_config(width=2048, blocks=2, vocab=32000, heads=16, dim=128, rot_dim=64, vdim=128, kv_rank=512, q_rank=768, experts=32, identity=2, top=6, ff=1408,
+                   taps=4, groups=8):
+    """`blocks` x (three latent-attention layers with direct queries, one with latent queries, YaRN rotation and head gates), each with a
+    mixture of experts behind it"""
+    mlp = {"kind": "moe", "expert": {"ff": ff}, "router": {"experts": experts, "identity": identity, "top": top}}
+    scale = float((dim + rot_dim) ** -0.5)
+    two = {"type": "latent_attention_2", "mixer": {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "scale": scale,
+                                                   "rot": {"base": 10000.0, "dims": rot_dim}}, "mlp": mlp}
+    one = {"type": "latent_attention", "mixer": {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "q_rank": q_rank, "scale": scale,
+                                                 "rot": {"base": 10000.0, "dims": rot_dim, "scaling": {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0}}},
+           "mlp": mlp}
+    return {"architecture": "Muzopel", "width": width, "vocab": vocab, "norm": {"eps": 1e-6, "groups": groups}, "canon": {"taps": taps}, "logit_softcap": 30.0,
+            "layers": [two, two, two, one] * blocks}
+
+
+def muzopel_tensor_shapes(cfg):
+    W_, V = cfg["width"], cfg["vocab"]
+    taps = cfg.get("canon", {}).get("taps", 0)
+    s = {"embed": (V, W_), "embed.norm": (W_,), "final.norm": (W_,), "head": (V, W_)}
+    for li, L in enumerate(cfg["layers"]):
+        p, m = "l%d." % li, L["mixer"]
+        H, dn, dr, dv, R = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
+        s[p + "norm1"] = (W_,); s[p + "dwa"] = (li + 2,)
+        if taps:
+            s[p + "canon1"] = (W_, taps)
+        if L["type"] == "latent_attention":
+            s.update({p + "mix.dq": (m["q_rank"], W_), p + "mix.dq.norm": (m["q_rank"],), p + "mix.uq": (H * (dn + dr), m["q_rank"]), p + "mix.g": (H, W_)})
+        else:
+            s[p + "mix.q"] = (H * (dn + dr), W_)
+        s.update({p + "mix.dkv": (R + dr, W_), p + "mix.dkv.norm": (R,), p + "mix.uk": (H * dn, R), p + "mix.uv": (H * dv, R), p + "mix.o": (W_, H * dv)})
+        if L.get("mlp"):
+            r, F = L["mlp"]["router"], L["mlp"]["expert"]["ff"]
+            s[p + "norm2"] = (W_,)
+            if taps:
+                s[p + "canon2"] = (W_, taps)
+            s[p + "mlp.router"] = (r["experts"] + r.get("identity", 0), W_); s[p + "mlp.correction"] = (r["experts"] + r.get("identity", 0),)
+            for e in range(r["experts"]):
+                s[p + "mlp.e%d.up" % e] = (F, W_); s[p + "mlp.e%d.down" % e] = (W_, F)
+    return s
+
+
+def write_muzopel_dir(path, cfg, seed=0):
+    return write_gelarax_dir(path, cfg, seed, muzopel_tensor_shapes(cfg))
+
+
+def write_gelarax_dir(path, cfg, seed=0, shapes=None):
     """config.json + model.safetensors (bfloat16, N(0, 1/fan_in) matrices, norm weights and layer scales near 1) for measurements"""
     import json
     import os
@@ -178,7 +223,8 @@ def write_gelarax_dir(path, cfg, seed=0):
     with open(os.path.join(path, "config.json"), "w") as f:
         json.dump(cfg, f)
     rng = np.random.default_rng(seed)
-    shapes = gelarax_tensor_shapes(cfg)
+    if shapes is None:
+        shapes = gelarax_tensor_shapes(cfg)
     header, off = {}, 0
     for name, shape in shapes.items():
         n = int(np.prod(shape)) * 2
@@ -190,8 +236,14 @@ def write_gelarax_dir(path, cfg, seed=0):
         f.write(struct.pack("<Q", len(hj))); f.write(hj)
         for name, shape in shapes.items():
             leaf = name.split(".")[-1]
-            if len(shape) == 1 and leaf in ("norm1", "norm", "ls1", "ls2"):
+            if len(shape) == 1 and leaf in ("norm1", "norm2", "norm", "ls1", "ls2"):
                 a = 1.0 + 0.05 * rng.standard_normal(shape, dtype=np.float32)
+            elif leaf == "dwa":
+                a = np.full(shape, 1.0 / shape[0], np.float32)
+            elif leaf == "correction":
+                a = 0.01 * rng.standard_normal(shape, dtype=np.float32)
+            elif leaf in ("canon1", "canon2"):
+                a = 0.2 * rng.standard_normal(shape, dtype=np.float32)
             elif leaf == "A_log":
                 a = rng.uniform(-3.0, 0.0, shape).astype(np.float32)
             elif len(shape) == 1 or leaf in ("rel", "conv"):
