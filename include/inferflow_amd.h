@@ -520,7 +520,7 @@ int ifa_kv_store_f32(const void *k_f32, size_t ldk, const void *v_f32, size_t ld
 /* softmax attention of the step's rows over their sequences' caches: query i sees key j iff j <= i and (i - j < window or
  * j < keep_first); q RMS-normed per head if norm_q; score = q.k * scale, soft cap cap * tanh(score / cap) if softcap > 0, + bias
  * rel[bucket_of[i - j]][head] if rel (bf16 [n_buckets][heads], bucket_of_dev: int per distance 0 .. max_ctx - 1); sink_bf16 [heads]
- * (nullable): exp(sink) joins the denominator.  dim <= 640.  out fp32 [rows][heads * dim].
+ * (nullable): exp(sink) joins the denominator.  dim <= 1024.  out fp32 [rows][heads * dim].
  * Steps of at least tile_min_rows rows (head sizes 32 / 64 / 96 / 128) take the tiled kernel -- 128 queries of one sequence per workgroup,
  * scores and weighted sums on the fp32 matrix cores -- which needs the step's sequences on the host too (seqs_host [n_seqs], the same
  * values as seqs_dev; NULL / n_seqs 0: always one workgroup per row).  With a workspace (ws_f32, ws_bytes; nullable) and at most 512
@@ -558,6 +558,13 @@ int ifa_latent_prepare_f32(const void *kv_f32, size_t ldkv, int kv_rank, int rot
 /* absorbed query: qa[t][h] = [W_uk[h]^T q_u[t][h] (kv_rank) | q_r[t][h] (rot_dim)]: a query against the cache rows themselves */
 int ifa_latent_absorb_q_f32(const void *q_f32, size_t ldq, int heads, int dim, int rot_dim, int kv_rank, const void *w_uk_bf16, size_t rows,
                             void *qa_f32, size_t ldqa, ifa_stream stream);
+/* single tokens: softmax attention of the absorbed queries over the cache rows of their sequences (keys: the whole row, values: its first
+ * kv_rank floats; causal); four heads share one read of the keys; the keys of a row are shared out to up to 64 workgroups per head group
+ * (max_keys = the longest sequence the cache holds sizes the shares) whose partial results go through ws_f32 (rows * heads * shares *
+ * (kv_rank + 2) floats at most).  kv_rank <= 1024.  out fp32 [rows][heads * kv_rank]. */
+int ifa_attention_latent_rows_f32(const void *qa_f32, size_t ldqa, int heads, int kv_rank, int rot_dim, float scale, const void *seqs_dev,
+                                  const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t cache_off, int max_keys, void *ws_f32,
+                                  size_t ws_bytes, void *out_f32, size_t ldo, ifa_stream stream);
 /* out[t][h * vdim + e] = gate[t][h] * sum_r w_uv[h * vdim + e][r] * ol[t][h * ld_head + r]; gate = sigmoid(g[t][h]) or 1 (g null) */
 int ifa_latent_expand_out_f32(const void *ol_f32, size_t ldol, int ld_head, int heads, int vdim, int kv_rank, const void *w_uv_bf16,
                               const void *g_f32, size_t ldg, size_t rows, void *out_f32, size_t ldo, ifa_stream stream);

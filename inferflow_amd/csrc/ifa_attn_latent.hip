@@ -56,42 +56,190 @@ __global__ void __launch_bounds__(256) k_latent_prepare(const float *__restrict_
     }
 }
 
-// grid (rows, heads): qa[t][h] = [sum_d q_u[d] W_uk[h * dim + d][r], r < R | q_r]
+// grid (rows, heads, chunks of 64 latent channels), four waves: qa[t][h][r] = sum_d q_u[d] W_uk[h * dim + d][r].  Lane = channel r (the
+// matrix rows are read coalesced), wave w sums a quarter of the d range, the quarters meet in LDS.  Chunk 0 also copies q_r behind.
 __global__ void __launch_bounds__(256) k_latent_absorb_q(const float *__restrict__ q, size_t ldq, int dim, int dr, int R, const bf16_t *__restrict__ wuk,
                                                          float *__restrict__ qa, size_t ldqa)
 {
-    extern __shared__ float qs[];          // [dim]
-    const int t = blockIdx.x, h = blockIdx.y;
+    __shared__ float part[4][64];
+    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const float *qh = q + (size_t)t * ldq + (size_t)h * (dim + dr);
     float *out = qa + (size_t)t * ldqa + (size_t)h * (R + dr);
-    for (int d = threadIdx.x; d < dim; d += blockDim.x) qs[d] = qh[d];
-    __syncthreads();
-    const bf16_t *w = wuk + (size_t)h * dim * R;
-    for (int r = threadIdx.x; r < R; r += blockDim.x) {
-        float acc = 0.0f;
-        for (int d = 0; d < dim; d++) acc = fmaf(qs[d], bf2f(w[(size_t)d * R + r]), acc);
-        out[r] = acc;
+    const int r = blockIdx.z * 64 + lane, dq = (dim + 3) / 4, d0 = wave * dq, d1 = min(dim, d0 + dq);
+    const bf16_t *w = wuk + (size_t)h * dim * R + r;
+    float acc = 0.0f;
+    if (r < R) {
+#pragma unroll 8
+        for (int d = d0; d < d1; d++) acc = fmaf(qh[d], bf2f(w[(size_t)d * R]), acc);
     }
-    for (int e = threadIdx.x; e < dr; e += blockDim.x) out[R + e] = qh[dim + e];
+    part[wave][lane] = acc;
+    __syncthreads();
+    if (wave == 0 && r < R) out[r] = (part[0][lane] + part[1][lane]) + (part[2][lane] + part[3][lane]);
+    if (blockIdx.z == 0) for (int e = threadIdx.x; e < dr; e += blockDim.x) out[R + e] = qh[dim + e];
 }
 
-// grid (rows, heads): out[t][h * vdim + e] = gate * sum_r W_uv[h * vdim + e][r] ol[t][h * ld_head + r]; a wave per e at a time
-__global__ void __launch_bounds__(256) k_latent_expand_out(const float *__restrict__ ol, size_t ldol, int ld_head, int vdim, int R, const bf16_t *__restrict__ wuv,
-                                                           const float *__restrict__ g, size_t ldg, float *__restrict__ out, size_t ldo)
+// grid (rows, groups of four output columns), a wave per column c = h * vdim + e: out[t][c] = gate[t][h] * sum_r W_uv[c][r] ol[t][h * ld_head + r]
+__global__ void __launch_bounds__(256) k_latent_expand_out(const float *__restrict__ ol, size_t ldol, int ld_head, int heads, int vdim, int R, const bf16_t *__restrict__ wuv,
+                                                           const float *__restrict__ g, size_t ldg, float *__restrict__ out, size_t ldo, int vec)
 {
-    extern __shared__ float os[];          // [R]
-    const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const int t = blockIdx.x, lane = threadIdx.x & 63, c = blockIdx.y * 4 + (threadIdx.x >> 6);
+    if (c >= heads * vdim) return;
+    const int h = c / vdim;
     const float *src = ol + (size_t)t * ldol + (size_t)h * ld_head;
-    for (int r = threadIdx.x; r < R; r += blockDim.x) os[r] = src[r];
-    __syncthreads();
-    const float gate = g ? sigmoid_f(g[(size_t)t * ldg + h]) : 1.0f;
-    for (int e = wave; e < vdim; e += nw) {
-        const bf16_t *w = wuv + ((size_t)h * vdim + e) * R;
-        float acc = 0.0f;
-        for (int r = lane; r < R; r += 64) acc = fmaf(bf2f(w[r]), os[r], acc);
-        acc = wave_sum(acc);
-        if (lane == 0) out[(size_t)t * ldo + (size_t)h * vdim + e] = acc * gate;
+    const bf16_t *w = wuv + (size_t)c * R;
+    float acc = 0.0f;
+    if (vec) {
+        for (int r = lane * 8; r < R; r += 512) {
+            const uint4 wv = *reinterpret_cast<const uint4 *>(w + r);
+            const float4 a0 = *reinterpret_cast<const float4 *>(src + r), a1 = *reinterpret_cast<const float4 *>(src + r + 4);
+            acc = fmaf(a0.x, __uint_as_float(wv.x << 16), acc); acc = fmaf(a0.y, __uint_as_float(wv.x & 0xFFFF0000u), acc);
+            acc = fmaf(a0.z, __uint_as_float(wv.y << 16), acc); acc = fmaf(a0.w, __uint_as_float(wv.y & 0xFFFF0000u), acc);
+            acc = fmaf(a1.x, __uint_as_float(wv.z << 16), acc); acc = fmaf(a1.y, __uint_as_float(wv.z & 0xFFFF0000u), acc);
+            acc = fmaf(a1.z, __uint_as_float(wv.w << 16), acc); acc = fmaf(a1.w, __uint_as_float(wv.w & 0xFFFF0000u), acc);
+        }
+    } else {
+        for (int r = lane; r < R; r += 64) acc = fmaf(bf2f(w[r]), src[r], acc);
     }
+    acc = wave_sum(acc);
+    if (lane == 0) out[(size_t)t * ldo + c] = g ? acc * sigmoid_f(g[(size_t)t * ldg + h]) : acc;
+}
+
+// ---- single tokens, absorbed form: the cache rows are keys (kv_rank + rot_dim) and values (the first kv_rank) of ONE head that all
+// query heads share.  grid (rows, groups of HB heads, key shares), four waves: a wave walks chunks of 16 keys, four lanes per key for the
+// scores of its HB heads (the key row is read ONCE for all of them, the queries sit in LDS), one value column per lane and CPL columns per
+// lane for the weighted sums, online softmax per head; the waves meet in LDS and leave {maximum, sum, weighted values} per share, which
+// k_attn_latent_rows_combine merges.  Scores, weights and sums are fp32.
+struct LatRowArgs {
+    const float *q; size_t ldq;                 // absorbed queries [rows][heads * (R + dr)]
+    int heads, R, dr;
+    float scale;
+    const SeqDesc *seqs; const int *row_seq; float *const *slot_base; size_t cache_off;
+    float *ws; int nsplit;                      // [rows][heads][nsplit][R + 2]
+    float *out; size_t ldo;                     // [rows][heads * R]
+    int vec;
+};
+
+template <int HB, int CPL>
+__global__ void __launch_bounds__(256) k_attn_latent_rows(LatRowArgs P)
+{
+    extern __shared__ float sm[];
+    const int D = P.R + P.dr, dv = P.R;
+    float *qs = sm;                              // [HB][D]
+    float *wm = qs + HB * D, *wl = wm + 4 * HB;  // [4][HB] each
+    float *wacc = wl + 4 * HB;                   // [4][HB][dv]
+    const int t = blockIdx.x, h0 = blockIdx.y * HB, split = blockIdx.z, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int nh = min(HB, P.heads - h0);
+    const SeqDesc sd = P.seqs[P.row_seq[t]];
+    const int i = sd.pos0 + t - sd.row0, nk = i + 1;
+    for (int e = tid; e < HB * D; e += blockDim.x) {
+        const int hh = e / D, c = e - hh * D;
+        qs[e] = hh < nh ? P.q[(size_t)t * P.ldq + (size_t)(h0 + hh) * D + c] : 0.0f;
+    }
+    __syncthreads();
+    const float *kc = P.slot_base[sd.slot] + P.cache_off;
+    float m[HB], l[HB], acc[HB][CPL];
+#pragma unroll
+    for (int hh = 0; hh < HB; hh++) {
+        m[hh] = -INFINITY; l[hh] = 0.0f;
+#pragma unroll
+        for (int e = 0; e < CPL; e++) acc[hh][e] = 0.0f;
+    }
+    const int nchunks = (nk + 15) / 16, sub = lane & 3;
+    for (int ch = split * 4 + wave; ch < nchunks; ch += 4 * P.nsplit) {
+        const int vi = ch * 16 + (lane >> 2);
+        const bool valid = vi < nk;
+        const float *kr = kc + (size_t)(valid ? vi : i) * D;
+        float s[HB];
+#pragma unroll
+        for (int hh = 0; hh < HB; hh++) s[hh] = 0.0f;
+        if (P.vec) {
+            for (int c = 4 * sub; c < D; c += 16) {
+                const float4 kv = *reinterpret_cast<const float4 *>(kr + c);
+#pragma unroll
+                for (int hh = 0; hh < HB; hh++) {
+                    const float *qq = qs + hh * D + c;
+                    s[hh] = fmaf(qq[0], kv.x, s[hh]); s[hh] = fmaf(qq[1], kv.y, s[hh]); s[hh] = fmaf(qq[2], kv.z, s[hh]); s[hh] = fmaf(qq[3], kv.w, s[hh]);
+                }
+            }
+        } else {
+            for (int c = sub; c < D; c += 4) {
+                const float kv = kr[c];
+#pragma unroll
+                for (int hh = 0; hh < HB; hh++) s[hh] = fmaf(qs[hh * D + c], kv, s[hh]);
+            }
+        }
+        float p[HB];
+#pragma unroll
+        for (int hh = 0; hh < HB; hh++) {
+            const float sc = valid ? quad_sum(s[hh]) * P.scale : -INFINITY;
+            const float m_new = fmaxf(m[hh], wave_max(sc));          // finite: the chunk holds at least one visible key
+            p[hh] = valid ? expf(sc - m_new) : 0.0f;
+            const float corr = m[hh] == -INFINITY ? 0.0f : expf(m[hh] - m_new);
+            l[hh] = l[hh] * corr + wave_sum(sub == 0 ? p[hh] : 0.0f);
+#pragma unroll
+            for (int e = 0; e < CPL; e++) acc[hh][e] *= corr;
+            m[hh] = m_new;
+        }
+        const int cnt = min(16, nk - ch * 16);
+        for (int jj = 0; jj < cnt; jj++) {
+            const float *vr = kc + (size_t)(ch * 16 + jj) * D;
+            float v[CPL];
+#pragma unroll
+            for (int e = 0; e < CPL; e++) { const int d = lane + 64 * e; v[e] = d < dv ? vr[d] : 0.0f; }
+#pragma unroll
+            for (int hh = 0; hh < HB; hh++) {
+                const float pj = __shfl(p[hh], 4 * jj, 64);
+#pragma unroll
+                for (int e = 0; e < CPL; e++) acc[hh][e] = fmaf(pj, v[e], acc[hh][e]);
+            }
+        }
+    }
+#pragma unroll
+    for (int hh = 0; hh < HB; hh++) {
+        if (lane == 0) { wm[wave * HB + hh] = m[hh]; wl[wave * HB + hh] = l[hh]; }
+#pragma unroll
+        for (int e = 0; e < CPL; e++) { const int d = lane + 64 * e; if (d < dv) wacc[(size_t)(wave * HB + hh) * dv + d] = acc[hh][e]; }
+    }
+    __syncthreads();
+    for (int hh = 0; hh < nh; hh++) {
+        float M = -INFINITY;
+        for (int w = 0; w < 4; w++) M = fmaxf(M, wm[w * HB + hh]);
+        float L = 0.0f, f[4];
+        for (int w = 0; w < 4; w++) { f[w] = wm[w * HB + hh] == -INFINITY ? 0.0f : expf(wm[w * HB + hh] - M); L += wl[w * HB + hh] * f[w]; }
+        float *dst = P.ws + (((size_t)t * P.heads + h0 + hh) * P.nsplit + split) * (dv + 2);
+        if (tid == 0) { dst[0] = M; dst[1] = L; }
+        for (int d = tid; d < dv; d += blockDim.x) {
+            float o = 0.0f;
+            for (int w = 0; w < 4; w++) o = fmaf(wacc[(size_t)(w * HB + hh) * dv + d], f[w], o);
+            dst[2 + d] = o;
+        }
+    }
+}
+
+// grid (rows, heads), one wave: lane sp holds share sp's maximum and sum (at most 64 shares)
+__global__ void __launch_bounds__(64) k_attn_latent_rows_combine(LatRowArgs P)
+{
+    const int t = blockIdx.x, h = blockIdx.y, dv = P.R, nsplit = P.nsplit, lane = threadIdx.x;
+    const float *src = P.ws + ((size_t)t * P.heads + h) * nsplit * (dv + 2);
+    const float m_sp = lane < nsplit ? src[(size_t)lane * (dv + 2)] : -INFINITY, l_sp = lane < nsplit ? src[(size_t)lane * (dv + 2) + 1] : 0.0f;
+    const float M = wave_max(m_sp);
+    const float f_sp = m_sp == -INFINITY ? 0.0f : expf(m_sp - M);
+    const float L = wave_sum(l_sp * f_sp);
+    for (int d = lane; d < dv; d += 64) {
+        float o = 0.0f;
+        for (int sp = 0; sp < nsplit; sp++) o = fmaf(src[(size_t)sp * (dv + 2) + 2 + d], __shfl(f_sp, sp, 64), o);
+        P.out[(size_t)t * P.ldo + (size_t)h * dv + d] = o / L;
+    }
+}
+
+constexpr int LR_HB = 4, LR_MAX_SPLITS = 64;
+
+template <int CPL>
+void launch_latent_rows(const LatRowArgs &P, unsigned rows, hipStream_t s)
+{
+    const size_t smem = ((size_t)LR_HB * (P.R + P.dr) + 8 * LR_HB + (size_t)4 * LR_HB * P.R) * 4;
+    if (smem > 48 * 1024) (void)hipFuncSetAttribute((const void *)k_attn_latent_rows<LR_HB, CPL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    hipLaunchKernelGGL((k_attn_latent_rows<LR_HB, CPL>), dim3(rows, (unsigned)((P.heads + LR_HB - 1) / LR_HB), (unsigned)P.nsplit), dim3(256), smem, s, P);
 }
 
 // ---- prompts: 128 queries of one sequence per workgroup, the keys 0 .. last query walked in blocks of 32 staged once per workgroup in
@@ -296,8 +444,9 @@ int ifa_latent_absorb_q_f32(const void *q_f32, size_t ldq, int heads, int dim, i
     IFA_REQUIRE(q_f32 && w_uk_bf16 && qa_f32, "ifa_latent_absorb_q_f32: null pointer");
     IFA_REQUIRE(heads > 0 && heads < 65536 && dim > 0 && dim <= 8192 && rot_dim >= 0 && kv_rank > 0 && rows > 0 && ldq >= (size_t)heads * (dim + rot_dim)
                 && ldqa >= (size_t)heads * (kv_rank + rot_dim), "ifa_latent_absorb_q_f32: bad shape");
-    hipLaunchKernelGGL(k_latent_absorb_q, dim3((unsigned)rows, (unsigned)heads), dim3(256), (size_t)dim * 4, ifa_s(stream), (const float *)q_f32, ldq, dim, rot_dim,
-                       kv_rank, (const bf16_t *)w_uk_bf16, (float *)qa_f32, ldqa);
+    IFA_REQUIRE(kv_rank <= 64 * 65535, "ifa_latent_absorb_q_f32: latent of %d channels", kv_rank);
+    hipLaunchKernelGGL(k_latent_absorb_q, dim3((unsigned)rows, (unsigned)heads, ifa_cdiv((size_t)kv_rank, 64)), dim3(256), 0, ifa_s(stream), (const float *)q_f32, ldq, dim,
+                       rot_dim, kv_rank, (const bf16_t *)w_uk_bf16, (float *)qa_f32, ldqa);
     IFA_LAUNCH_CHECK();
     return IFA_OK;
 }
@@ -308,8 +457,42 @@ int ifa_latent_expand_out_f32(const void *ol_f32, size_t ldol, int ld_head, int 
     IFA_REQUIRE(ol_f32 && w_uv_bf16 && out_f32, "ifa_latent_expand_out_f32: null pointer");
     IFA_REQUIRE(heads > 0 && heads < 65536 && vdim > 0 && kv_rank > 0 && kv_rank <= 8192 && ld_head >= kv_rank && rows > 0 && ldol >= (size_t)(heads - 1) * ld_head + kv_rank
                 && ldo >= (size_t)heads * vdim && (!g_f32 || ldg >= (size_t)heads), "ifa_latent_expand_out_f32: bad shape");
-    hipLaunchKernelGGL(k_latent_expand_out, dim3((unsigned)rows, (unsigned)heads), dim3(256), (size_t)kv_rank * 4, ifa_s(stream), (const float *)ol_f32, ldol, ld_head,
-                       vdim, kv_rank, (const bf16_t *)w_uv_bf16, (const float *)g_f32, ldg, (float *)out_f32, ldo);
+    IFA_REQUIRE((size_t)heads * vdim <= 4 * 65535, "ifa_latent_expand_out_f32: %d x %d output columns", heads, vdim);
+    // 16-byte requests: whole 8-element pieces in every matrix row, every head's part of a latent row on a 16-byte boundary
+    const int vec = (kv_rank % 8 == 0 && ld_head % 4 == 0 && ldol % 4 == 0 && ((uintptr_t)ol_f32 & 15) == 0 && ((uintptr_t)w_uv_bf16 & 15) == 0) ? 1 : 0;
+    hipLaunchKernelGGL(k_latent_expand_out, dim3((unsigned)rows, ifa_cdiv((size_t)heads * vdim, 4)), dim3(256), 0, ifa_s(stream), (const float *)ol_f32, ldol, ld_head,
+                       heads, vdim, kv_rank, (const bf16_t *)w_uv_bf16, (const float *)g_f32, ldg, (float *)out_f32, ldo, vec);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_attention_latent_rows_f32(const void *qa_f32, size_t ldqa, int heads, int kv_rank, int rot_dim, float scale, const void *seqs_dev,
+                                  const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t cache_off, int max_keys, void *ws_f32,
+                                  size_t ws_bytes, void *out_f32, size_t ldo, ifa_stream stream)
+{
+    IFA_REQUIRE(qa_f32 && seqs_dev && row_seq_dev && slot_base_dev && ws_f32 && out_f32, "ifa_attention_latent_rows_f32: null pointer");
+    IFA_REQUIRE(heads > 0 && heads < 65536 * LR_HB && kv_rank > 0 && kv_rank <= 1024 && rot_dim >= 0 && rows > 0 && rows < 65536 && max_keys >= 1
+                && ldqa >= (size_t)heads * (kv_rank + rot_dim) && ldo >= (size_t)heads * kv_rank, "ifa_attention_latent_rows_f32: bad shape");
+    LatRowArgs P;
+    P.q = (const float *)qa_f32; P.ldq = ldqa; P.heads = heads; P.R = kv_rank; P.dr = rot_dim; P.scale = scale; P.seqs = (const SeqDesc *)seqs_dev;
+    P.row_seq = row_seq_dev; P.slot_base = (float *const *)slot_base_dev; P.cache_off = cache_off; P.ws = (float *)ws_f32; P.out = (float *)out_f32; P.ldo = ldo;
+    P.vec = ((kv_rank + rot_dim) % 4 == 0 && cache_off % 4 == 0) ? 1 : 0;
+    // key shares: 64 keys a share over the longest sequence the cache holds (the same for every step, so that a captured step replays),
+    // fewer where many rows already fill the chip or the workspace is small
+    int nsplit = std::min(LR_MAX_SPLITS, (max_keys + 63) / 64);
+    const size_t groups = (size_t)(heads + LR_HB - 1) / LR_HB;
+    while (nsplit > 1 && rows * groups * (size_t)nsplit > 2048) nsplit--;
+    while (nsplit > 1 && rows * (size_t)heads * nsplit * ((size_t)kv_rank + 2) * 4 > ws_bytes) nsplit--;
+    IFA_REQUIRE(rows * (size_t)heads * nsplit * ((size_t)kv_rank + 2) * 4 <= ws_bytes, "ifa_attention_latent_rows_f32: workspace of %zu bytes is too small", ws_bytes);
+    P.nsplit = nsplit;
+    hipStream_t s = ifa_s(stream);
+    const int cpl = (kv_rank + 63) / 64;
+    if (cpl <= 1) launch_latent_rows<1>(P, (unsigned)rows, s);
+    else if (cpl <= 2) launch_latent_rows<2>(P, (unsigned)rows, s);
+    else if (cpl <= 4) launch_latent_rows<4>(P, (unsigned)rows, s);
+    else if (cpl <= 8) launch_latent_rows<8>(P, (unsigned)rows, s);
+    else launch_latent_rows<16>(P, (unsigned)rows, s);
+    hipLaunchKernelGGL(k_attn_latent_rows_combine, dim3((unsigned)rows, (unsigned)heads), dim3(64), 0, s, P);
     IFA_LAUNCH_CHECK();
     return IFA_OK;
 }

@@ -47,7 +47,7 @@ struct WinAttnArgs {
     float *ws; int nsplit;           // nsplit > 1: the keys of a (row, head) are shared out to nsplit workgroups; partial results in ws [rows][heads][nsplit][dim + 2]
 };
 
-constexpr int WA_DPL_MAX = 10;    // dim <= 64 * DPL: a lane holds DPL value columns (1, 2, 4 or 10: up to 640, the row of a latent-attention cache)
+constexpr int WA_DPL_MAX = 16;    // dim <= 64 * DPL: a lane holds DPL value columns (1, 2, 4, 10 or 16: up to 1024, the row of a latent-attention cache)
 
 // grid (rows, heads, splits), four waves: the visible keys (kept first tokens, then the window) are walked in chunks of 16, four
 // lanes per key for the score, one value column per lane for the weighted sum; chunks go round-robin to the waves, each
@@ -364,6 +364,7 @@ int ifa_attention_window_f32(const void *q_f32, size_t ldq, int heads, int kv_he
     if (dim <= 64) hipLaunchKernelGGL(k_attn_window<1>, grid_rows, dim3(256), smem, ifa_s(stream), P);
     else if (dim <= 128) hipLaunchKernelGGL(k_attn_window<2>, grid_rows, dim3(256), smem, ifa_s(stream), P);
     else if (dim <= 256) hipLaunchKernelGGL(k_attn_window<4>, grid_rows, dim3(256), smem, ifa_s(stream), P);
+    else if (dim <= 640) hipLaunchKernelGGL(k_attn_window<10>, grid_rows, dim3(256), smem, ifa_s(stream), P);
     else hipLaunchKernelGGL(k_attn_window<WA_DPL_MAX>, grid_rows, dim3(256), smem, ifa_s(stream), P);
     if (nsplit > 1) hipLaunchKernelGGL(k_attn_window_combine, dim3((unsigned)rows, (unsigned)heads), dim3(64), 0, ifa_s(stream), P);
     IFA_LAUNCH_CHECK();

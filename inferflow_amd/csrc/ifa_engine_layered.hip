@@ -214,6 +214,16 @@ int ensure_rows(ifa_model *m, size_t T, size_t nseq)
         const size_t W = (size_t)n->cfg.width;
         const size_t sz[] = {W, W, n->n_in_max, n->mix_max, n->mix_max, std::max<size_t>(n->ffn_max, 4), std::max<size_t>(n->heads_max, 4), std::max<size_t>(n->heads_max, 4)};
         for (size_t i = 0; i < 8; i++) IFA_HIP_CHECK(hipMalloc((void **)bufs[i], T * sz[i] * 4));
+        {   // the single-row latent attention leaves at least one partial result per (row, head) in the workspace
+            size_t need = 0;
+            for (const LLayer &L : n->layers)
+                if (L.spec.mixer == IFA_MIX_LATENT) need = std::max(need, T * (size_t)L.spec.m_heads * ((size_t)L.spec.m_kv_rank + 2) * 4);
+            if (need > n->attn_ws_bytes) {
+                lay_free(n->attn_ws); n->attn_ws = nullptr;
+                IFA_HIP_CHECK(hipMalloc((void **)&n->attn_ws, need));
+                n->attn_ws_bytes = need;
+            }
+        }
         lay_free(n->m4); lay_free(n->m5); lay_free(n->stack); lay_free(n->moe_wgt); lay_free(n->moe_idx); lay_free(n->moe_ws);
         n->m4 = n->m5 = n->stack = n->moe_wgt = nullptr; n->moe_idx = nullptr; n->moe_ws = nullptr; n->moe_ws_bytes = 0;
         if (n->any_latent) { IFA_HIP_CHECK(hipMalloc((void **)&n->m4, T * n->mix_max * 4)); IFA_HIP_CHECK(hipMalloc((void **)&n->m5, T * n->mix_max * 4)); }
@@ -293,12 +303,12 @@ int run_postnorm_layer(ifa_model *m, LLayer &L, size_t li, size_t T, int nseq)
             if ((rc = ifa_attention_latent_tile_f32(q, ldq, H, dn, dr, dv, R, sp.m_scale, n->kx, ldk, n->vx, ldv, n->ctx0_dev, gate, NI, n->seqs_dev, n->seqs_host.data(),
                                                     (int)n->seqs_host.size(), slots, L.o_c, n->m5, OV, s))) return rc;
         } else {
-            // absorbed form: the cache rows are keys and values of ONE shared head of kv_rank + rot_dim dimensions
+            // absorbed form: the cache rows are keys (whole) and values (latent part) of ONE head that all query heads share
             const size_t QA = (size_t)H * CR;
             if ((rc = ifa_latent_absorb_q_f32(q, ldq, H, dn, dr, R, L.T(IFA_LT_M_UK).data, T, n->m2, QA, s))) return rc;
-            if ((rc = ifa_attention_window_f32(n->m2, QA, H, 1, (int)CR, 0, c.eps, sp.m_scale, 0.0f, c.max_ctx, 0, nullptr, nullptr, 0, nullptr, n->seqs_dev, n->row_seq_dev,
-                                               T, slots, L.o_c, L.o_c, n->m4, QA, nullptr, 0, 1 << 30, n->attn_ws, n->attn_ws_bytes, s))) return rc;
-            if ((rc = ifa_latent_expand_out_f32(n->m4, QA, (int)CR, H, dv, R, L.T(IFA_LT_M_UV).data, gate, NI, T, n->m5, OV, s))) return rc;
+            if ((rc = ifa_attention_latent_rows_f32(n->m2, QA, H, R, dr, sp.m_scale, n->seqs_dev, n->row_seq_dev, T, slots, L.o_c, c.max_ctx, n->attn_ws, n->attn_ws_bytes,
+                                                    n->m4, (size_t)H * R, s))) return rc;
+            if ((rc = ifa_latent_expand_out_f32(n->m4, (size_t)H * R, R, H, dv, R, L.T(IFA_LT_M_UV).data, gate, NI, T, n->m5, OV, s))) return rc;
         }
         if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_M_O).data, W, OV, n->m5, OV, T, nullptr, nullptr, 1.0f, 0, n->m1, W))) return rc;
         if ((rc = ifa_group_rmsnorm_f32(n->m1, W, T, W, c.norm_groups, L.T(IFA_LT_NORM1).data, c.eps, 1, n->x, W, s))) return rc;
@@ -584,7 +594,7 @@ int lay_finalize(ifa_model *m)
         size_t per_row = 0;
         for (const LLayer &L : n->layers)
             if (L.spec.mixer == IFA_MIX_WINDOW_LINEAR) per_row = std::max(per_row, (size_t)L.spec.a_heads * 32 * ((size_t)L.spec.a_dim + 2) * 4);
-            else if (L.spec.mixer == IFA_MIX_LATENT) per_row = std::max(per_row, (size_t)L.spec.m_heads * 32 * ((size_t)(L.spec.m_kv_rank + L.spec.m_rot_dim) + 2) * 4);
+            else if (L.spec.mixer == IFA_MIX_LATENT) per_row = std::max(per_row, (size_t)L.spec.m_heads * 16 * ((size_t)L.spec.m_kv_rank + 2) * 4);
         n->attn_ws_bytes = per_row * 64;
         if (n->attn_ws_bytes) IFA_HIP_CHECK(hipMalloc((void **)&n->attn_ws, n->attn_ws_bytes));
     }
@@ -864,7 +874,7 @@ int ifa_model_create_layered(const ifa_layered_config *cfg, const ifa_layer_spec
             IFA_REQUIRE(s.d_heads > 0 && s.d_kv_heads > 0 && s.d_heads % s.d_kv_heads == 0 && s.d_dim > 0 && s.d_dim <= 256 && s.d_vdim > 0 && s.d_conv >= 1 && s.d_conv <= 64,
                         "ifa_model_create_layered: layer %d: bad delta-rule sizes", l);
         } else if (s.mixer == IFA_MIX_LATENT) {
-            IFA_REQUIRE(s.m_heads > 0 && s.m_dim > 0 && s.m_rot_dim >= 0 && s.m_vdim > 0 && s.m_kv_rank > 0 && s.m_q_rank >= 0 && s.m_kv_rank + s.m_rot_dim <= 640
+            IFA_REQUIRE(s.m_heads > 0 && s.m_dim > 0 && s.m_rot_dim >= 0 && s.m_vdim > 0 && s.m_kv_rank > 0 && s.m_q_rank >= 0 && s.m_kv_rank + s.m_rot_dim <= 1024
                         && s.m_rot_dims >= 0 && s.m_rot_dims <= s.m_rot_dim && s.m_rot_dims % 2 == 0 && (s.m_rot_dims == 0 || s.m_rot_base > 1.0f),
                         "ifa_model_create_layered: layer %d: bad latent-attention sizes", l);
             IFA_REQUIRE(s.m_yarn_factor == 0.0f || (s.m_yarn_factor > 0.0f && s.m_yarn_original > 0.0f && s.m_yarn_fast > 0.0f && s.m_yarn_slow > 0.0f),

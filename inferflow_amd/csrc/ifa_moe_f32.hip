@@ -60,6 +60,7 @@ __global__ void __launch_bounds__(256) k_moe_up_rows(const float *__restrict__ h
         const bf16_t *w = up + ((size_t)e * F + n) * W;
         float acc = 0.0f;
         if (vec) {
+#pragma unroll 4
             for (int k = lane * 8; k < W; k += 512) {
                 const u32x4m wv = *reinterpret_cast<const u32x4m *>(w + k);
                 const float4 a0 = *reinterpret_cast<const float4 *>(hr + k), a1 = *reinterpret_cast<const float4 *>(hr + k + 4);
@@ -76,7 +77,8 @@ __global__ void __launch_bounds__(256) k_moe_up_rows(const float *__restrict__ h
     }
 }
 
-// grid (width chunks, rows): y[t][c] (+)= sum_k wgt * (identity ? h[t][c] : W_down[e][c] . act[p]); a wave per c at a time
+// grid (width chunks, rows): y[t][c] (+)= sum_k wgt * (identity ? h[t][c] : W_down[e][c] . act[p]); a wave per c at a time.  The chosen
+// experts are walked eight at a time with their loads issued side by side (a step of one token is bound by requests in flight).
 __global__ void __launch_bounds__(256) k_moe_down_rows(const float *__restrict__ h, size_t ldh, int W, int F, int experts, int top, const bf16_t *__restrict__ down,
                                                        const int *__restrict__ idx, const float *__restrict__ wgt, const float *__restrict__ act,
                                                        int accumulate, float *__restrict__ y, size_t ldy, int vec)
@@ -85,26 +87,46 @@ __global__ void __launch_bounds__(256) k_moe_down_rows(const float *__restrict__
     const int lane = threadIdx.x & 63, wave = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6), nwaves = gridDim.x * (blockDim.x >> 6);
     for (int c = wave; c < W; c += nwaves) {
         float out = 0.0f;
-        for (int k = 0; k < top; k++) {
-            const int p = t * top + k, e = idx[p];
-            const float wk = wgt[p];
-            if (e >= experts) { out = fmaf(wk, h[(size_t)t * ldh + c], out); continue; }
-            const bf16_t *w = down + ((size_t)e * W + c) * F;
-            const float *a = act + (size_t)p * F;
-            float acc = 0.0f;
+        for (int k0 = 0; k0 < top; k0 += 8) {
+            int e[8]; float acc[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) { e[k] = k0 + k < top ? idx[t * top + k0 + k] : experts; acc[k] = 0.0f; }
             if (vec) {
                 for (int j = lane * 8; j < F; j += 512) {
-                    const u32x4m wv = *reinterpret_cast<const u32x4m *>(w + j);
-                    const float4 a0 = *reinterpret_cast<const float4 *>(a + j), a1 = *reinterpret_cast<const float4 *>(a + j + 4);
-                    acc = fmaf(a0.x, __uint_as_float(wv[0] << 16), acc); acc = fmaf(a0.y, __uint_as_float(wv[0] & 0xFFFF0000u), acc);
-                    acc = fmaf(a0.z, __uint_as_float(wv[1] << 16), acc); acc = fmaf(a0.w, __uint_as_float(wv[1] & 0xFFFF0000u), acc);
-                    acc = fmaf(a1.x, __uint_as_float(wv[2] << 16), acc); acc = fmaf(a1.y, __uint_as_float(wv[2] & 0xFFFF0000u), acc);
-                    acc = fmaf(a1.z, __uint_as_float(wv[3] << 16), acc); acc = fmaf(a1.w, __uint_as_float(wv[3] & 0xFFFF0000u), acc);
+                    u32x4m wv[8]; float4 a0[8], a1[8];
+#pragma unroll
+                    for (int k = 0; k < 8; k++)
+                        if (e[k] < experts) {
+                            wv[k] = *reinterpret_cast<const u32x4m *>(down + ((size_t)e[k] * W + c) * F + j);
+                            const float *a = act + (size_t)(t * top + k0 + k) * F + j;
+                            a0[k] = *reinterpret_cast<const float4 *>(a); a1[k] = *reinterpret_cast<const float4 *>(a + 4);
+                        }
+#pragma unroll
+                    for (int k = 0; k < 8; k++)
+                        if (e[k] < experts) {
+                            float s = acc[k];
+                            s = fmaf(a0[k].x, __uint_as_float(wv[k][0] << 16), s); s = fmaf(a0[k].y, __uint_as_float(wv[k][0] & 0xFFFF0000u), s);
+                            s = fmaf(a0[k].z, __uint_as_float(wv[k][1] << 16), s); s = fmaf(a0[k].w, __uint_as_float(wv[k][1] & 0xFFFF0000u), s);
+                            s = fmaf(a1[k].x, __uint_as_float(wv[k][2] << 16), s); s = fmaf(a1[k].y, __uint_as_float(wv[k][2] & 0xFFFF0000u), s);
+                            s = fmaf(a1[k].z, __uint_as_float(wv[k][3] << 16), s); s = fmaf(a1[k].w, __uint_as_float(wv[k][3] & 0xFFFF0000u), s);
+                            acc[k] = s;
+                        }
                 }
             } else {
-                for (int j = lane; j < F; j += 64) acc = fmaf(a[j], bf2f(w[j]), acc);
+#pragma unroll
+                for (int k = 0; k < 8; k++)
+                    if (e[k] < experts) {
+                        const bf16_t *w = down + ((size_t)e[k] * W + c) * F;
+                        const float *a = act + (size_t)(t * top + k0 + k) * F;
+                        for (int j = lane; j < F; j += 64) acc[k] = fmaf(a[j], bf2f(w[j]), acc[k]);
+                    }
             }
-            out = fmaf(wk, wave_sum(acc), out);
+#pragma unroll
+            for (int k = 0; k < 8; k++) {      // in the order of the row's choices
+                if (k0 + k >= top) break;
+                const float wk = wgt[t * top + k0 + k];
+                out = fmaf(wk, e[k] < experts ? wave_sum(acc[k]) : h[(size_t)t * ldh + c], out);
+            }
         }
         if (lane == 0) { float *d = y + (size_t)t * ldy + c; *d = accumulate ? *d + out : out; }
     }
@@ -206,9 +228,9 @@ int ifa_moe_experts_f32(const void *h_f32, size_t ldh, size_t rows, int width, i
         const int vec_u = (width % 8 == 0 && ldh % 4 == 0 && ((uintptr_t)h_f32 & 15) == 0 && ((uintptr_t)up_bf16 & 15) == 0) ? 1 : 0;
         const int vec_d = (ff % 8 == 0 && ((uintptr_t)down_bf16 & 15) == 0) ? 1 : 0;
         if (experts > 0)
-            hipLaunchKernelGGL(k_moe_up_rows, dim3(std::min(64u, ifa_cdiv((size_t)ff, 4)), (unsigned)pairs), dim3(256), 0, s, h, ldh, width, ff, experts, top,
+            hipLaunchKernelGGL(k_moe_up_rows, dim3(std::min(512u, ifa_cdiv((size_t)ff, 4)), (unsigned)pairs), dim3(256), 0, s, h, ldh, width, ff, experts, top,
                                (const bf16_t *)up_bf16, idx_dev, actb, vec_u);
-        hipLaunchKernelGGL(k_moe_down_rows, dim3(std::min(256u, ifa_cdiv((size_t)width, 4)), (unsigned)rows), dim3(256), 0, s, h, ldh, width, ff, experts, top,
+        hipLaunchKernelGGL(k_moe_down_rows, dim3(std::min(1024u, ifa_cdiv((size_t)width, 4)), (unsigned)rows), dim3(256), 0, s, h, ldh, width, ff, experts, top,
                            (const bf16_t *)down_bf16, idx_dev, (const float *)wgt_f32, actb, accumulate ? 1 : 0, (float *)y_f32, ldy, vec_d);
         IFA_LAUNCH_CHECK();
         return IFA_OK;

@@ -111,8 +111,10 @@ def latent_case(rng, H, dn, dr, dv, R, rot, first):
     return mx, P
 
 
-def run_latent(L, mx, P, q, kv, gate, seqs, slots, expanded, first, ops32=1):
-    """the worker's sequence of ops over one step; q [rows, H (dn + dr)], kv [rows, R + dr], gate [rows, H] or None"""
+def run_latent(L, mx, P, q, kv, gate, seqs, slots, expanded, first, ops32=1, window_kernel=False):
+    """the worker's sequence of ops over one step; q [rows, H (dn + dr)], kv [rows, R + dr], gate [rows, H] or None.  expanded: keys / values
+    from the cached latents + the tiled kernel; else the absorbed form through the head-sharing single-row kernel, or (window_kernel)
+    through the general single-row kernel with one shared KV head whose value row is its key row"""
     H, dn, dr, dv, R = mx["heads"], mx["dim"], mx["rot_dim"], mx["vdim"], mx["kv_rank"]
     CR, QD, OV = R + dr, H * (dn + dr), H * dv
     rot = dict(mx["rot"])
@@ -142,18 +144,25 @@ def run_latent(L, mx, P, q, kv, gate, seqs, slots, expanded, first, ops32=1):
         ia.check(L.ifa_attention_latent_tile_f32(p(qd), QD, H, dn, dr, dv, R, mx["scale"], p(kx), H * dn, p(vx), OV, p(devi(ctx0)), p(gd) if gd is not None else None, H,
                                                  p(sd), host.ctypes.data_as(C.c_void_p), len(seqs), p(slots.table), 0, p(out), OV, None))
     else:
-        qa = torch.zeros((rows, H * CR), dtype=torch.float32, device="cuda"); ol = torch.zeros_like(qa)
-        ws = torch.zeros(rows * H * 32 * (CR + 2), dtype=torch.float32, device="cuda")
+        qa = torch.zeros((rows, H * CR), dtype=torch.float32, device="cuda")
         ia.check(L.ifa_latent_absorb_q_f32(p(qd), QD, H, dn, dr, R, p(uk), rows, p(qa), H * CR, None))
-        ia.check(L.ifa_attention_window_f32(p(qa), H * CR, H, 1, CR, 0, 1e-6, mx["scale"], 0.0, 4096, 0, None, None, 0, None, p(sd), p(rs), rows, p(slots.table), 0, 0,
-                                            p(ol), H * CR, None, 0, 1 << 30, p(ws), ws.numel() * 4, None))
-        ia.check(L.ifa_latent_expand_out_f32(p(ol), H * CR, CR, H, dv, R, p(uv), p(gd) if gd is not None else None, H, rows, p(out), OV, None))
+        if window_kernel:
+            ol = torch.zeros_like(qa)
+            ws = torch.zeros(rows * H * 32 * (CR + 2), dtype=torch.float32, device="cuda")
+            ia.check(L.ifa_attention_window_f32(p(qa), H * CR, H, 1, CR, 0, 1e-6, mx["scale"], 0.0, 4096, 0, None, None, 0, None, p(sd), p(rs), rows, p(slots.table), 0, 0,
+                                                p(ol), H * CR, None, 0, 1 << 30, p(ws), ws.numel() * 4, None))
+            ia.check(L.ifa_latent_expand_out_f32(p(ol), H * CR, CR, H, dv, R, p(uv), p(gd) if gd is not None else None, H, rows, p(out), OV, None))
+        else:
+            ol = torch.zeros((rows, H * R), dtype=torch.float32, device="cuda")
+            ws = torch.zeros(rows * H * 8 * (R + 2), dtype=torch.float32, device="cuda")          # room for 8 key shares a row
+            ia.check(L.ifa_attention_latent_rows_f32(p(qa), H * CR, H, R, dr, mx["scale"], p(sd), p(rs), rows, p(slots.table), 0, 160, p(ws), ws.numel() * 4, p(ol), H * R, None))
+            ia.check(L.ifa_latent_expand_out_f32(p(ol), H * R, R, H, dv, R, p(uv), p(gd) if gd is not None else None, H, rows, p(out), OV, None))
     sync()
     return out.cpu().numpy()
 
 
 @pytest.mark.parametrize("H,dn,dr,dv,R,rdims,first", [(2, 16, 8, 24, 32, 8, True), (4, 32, 32, 80, 64, 32, False), (1, 5, 6, 7, 9, 4, True), (2, 128, 64, 128, 224, 64, False),
-                                                      (3, 48, 0, 16, 20, 0, False)])
+                                                      (3, 48, 0, 16, 20, 0, False), (6, 24, 16, 32, 600, 16, True), (9, 8, 4, 8, 144, 4, False)])
 def test_latent_attention_both_forms_whole_portions_and_several_sequences(H, dn, dr, dv, R, rdims, first):
     rng = np.random.default_rng(H * 100 + dn + R)
     rot = {"base": 500.0, "dims": rdims}
@@ -173,12 +182,12 @@ def test_latent_attention_both_forms_whole_portions_and_several_sequences(H, dn,
     slots = Slots(3, 160 * (R + dr) + 4)
     tol = 2e-5 * max(1.0, max(np.abs(d[3]).max() for d in data))
     # whole sequences in one step, in the tiled form and in the single-row form
-    for expanded in (True, False):
+    for expanded, window_kernel in ((True, False), (False, False), (False, True)):
         seqs = [(n, 0, i) for i, n in enumerate(lens)]
         q = np.concatenate([d[0] for d in data]); kv = np.concatenate([d[1] for d in data])
         g = np.concatenate([d[2] for d in data]) if first else None
-        got = run_latent(L, mx, P, q, kv, g, seqs, slots, expanded, first)
-        assert np.abs(got - np.concatenate([d[3] for d in data])).max() < tol, expanded
+        got = run_latent(L, mx, P, q, kv, g, seqs, slots, expanded, first, window_kernel=window_kernel)
+        assert np.abs(got - np.concatenate([d[3] for d in data])).max() < tol, (expanded, window_kernel)
     # the first two sequences in portions (slots swapped: reused), a prefix in one form and the rest in the other or token by token
     for (first_part, rest_expanded, step) in ((100, True, 50), (129, False, 1), (31, True, 33), (2, False, 1)):
         for si, slot in ((0, 1), (1, 0)):
