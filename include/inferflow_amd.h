@@ -540,6 +540,13 @@ int ifa_group_rmsnorm_f32(const void *x_f32, size_t ldx, size_t rows, size_t col
  * the last taps - 1 inputs carried in the slot like ifa_shortconv_silu_f32's (ifa_shortconv_tail_f32 advances them afterwards) */
 int ifa_shortconv_residual_f32(const void *x_f32, size_t ldx, int channels, int taps, const void *w_bf16, const void *seqs_dev, const int *row_seq_dev,
                                size_t rows, void *const *slot_base_dev, size_t state_off, void *y_f32, size_t ldy, ifa_stream stream);
+/* Steps of a few rows (<= 64; a workgroup per norm part): what lies between two sub-layers of a post-norm block in ONE launch, every part optional:
+ * x[t] += group_rms_norm(m[t]) * norm_w (m null: skip); depth average as ifa_depth_average_f32 (stack null: skip); h = x + conv(x) with the
+ * carried tail read and then advanced, as ifa_shortconv_residual_f32 + ifa_shortconv_tail_f32 (conv_w null: skip).  x is rows x cols, contiguous. */
+int ifa_norm_add_conv_rows_f32(void *x_f32, size_t rows, size_t cols, const void *m_f32, size_t ldm, const void *norm_w_bf16, int groups, float eps,
+                               void *stack_f32, size_t plane_stride, int count, const void *depth_w_bf16, const void *conv_w_bf16, int taps,
+                               const void *seqs_dev, int n_seqs, const int *row_seq_dev, void *const *slot_base_dev, size_t state_off, void *h_f32,
+                               ifa_stream stream);
 /* depth average: stack[count - 1] <- x (rows x cols, contiguous), then x <- sum_j w[j] stack[j], j < count; stack planes are
  * plane_stride floats apart; w bf16 [count] */
 int ifa_depth_average_f32(void *x_f32, size_t rows, size_t cols, void *stack_f32, size_t plane_stride, int count, const void *w_bf16, ifa_stream stream);
@@ -584,6 +591,9 @@ int ifa_attention_latent_tile_fits(int dim, int rot_dim, int vdim);
  * not renormalized.  idx_dev / wgt_dev: [rows][top]. */
 int ifa_moe_route_f32(const void *logits_f32, size_t ld, size_t rows, int n_all, int top, const void *correction_bf16, int *idx_dev, void *wgt_f32,
                       ifa_stream stream);
+/* the same for steps of at most 64 rows with the router's product (router_bf16 [n_all][width], fp32 dots) inside the launch */
+int ifa_moe_route_rows_f32(const void *h_f32, size_t ldh, size_t rows, int width, const void *router_bf16, int n_all, int top, const void *correction_bf16,
+                           int *idx_dev, void *wgt_f32, ifa_stream stream);
 /* y[t] (+)= sum_k wgt[t][k] * expert_{idx[t][k]}(h[t]); act 0: exact (erf) GELU.  Rows are served by expert: few rows stream each chosen
  * expert's weights per row; many rows are sorted by expert and run as grouped matrix-core products (ops32 as in ifa_linear_bf16w).
  * ws: workspace of ifa_moe_workspace_bytes(rows, top, width, ff, experts) bytes.  Deterministic: no atomics on values. */

@@ -166,6 +166,7 @@ SIGNATURES = {
     "ifa_embed_rows_f32": (_i, [_vp, _i, _i, _vp, _sz, _vp, _vp]),
     "ifa_group_rmsnorm_f32": (_i, [_vp, _sz, _sz, _sz, _i, _vp, _f, _i, _vp, _sz, _vp]),
     "ifa_shortconv_residual_f32": (_i, [_vp, _sz, _i, _i, _vp, _vp, _vp, _sz, _vp, _sz, _vp, _sz, _vp]),
+    "ifa_norm_add_conv_rows_f32": (_i, [_vp, _sz, _sz, _vp, _sz, _vp, _i, _f, _vp, _sz, _i, _vp, _vp, _i, _vp, _i, _vp, _vp, _sz, _vp, _vp]),
     "ifa_depth_average_f32": (_i, [_vp, _sz, _sz, _vp, _sz, _i, _vp, _vp]),
     "ifa_softcap_f32": (_i, [_vp, _sz, _f, _vp]),
     "ifa_latent_prepare_f32": (_i, [_vp, _sz, _i, _i, _i, _vp, _f, _vp, _sz, _i, _i, _vp, _f, _vp, _vp, _sz, _vp, _sz, _vp]),
@@ -175,6 +176,7 @@ SIGNATURES = {
     "ifa_attention_latent_tile_f32": (_i, [_vp, _sz, _i, _i, _i, _i, _i, _f, _vp, _sz, _vp, _sz, _vp, _vp, _sz, _vp, _vp, _i, _vp, _sz, _vp, _sz, _vp]),
     "ifa_attention_latent_tile_fits": (_i, [_i, _i, _i]),
     "ifa_moe_route_f32": (_i, [_vp, _sz, _sz, _i, _i, _vp, _vp, _vp, _vp]),
+    "ifa_moe_route_rows_f32": (_i, [_vp, _sz, _sz, _i, _vp, _i, _i, _vp, _vp, _vp, _vp]),
     "ifa_moe_workspace_bytes": (_sz, [_sz, _i, _i, _i, _i]),
     "ifa_moe_experts_f32": (_i, [_vp, _sz, _sz, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _sz, _vp, _sz, _i, _vp]),
     "ifa_model_create_layered": (_i, [_vp, _vp, C.POINTER(_vp)]),

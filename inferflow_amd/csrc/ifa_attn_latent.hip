@@ -216,7 +216,8 @@ __global__ void __launch_bounds__(256) k_attn_latent_rows(LatRowArgs P)
     }
 }
 
-// grid (rows, heads), one wave: lane sp holds share sp's maximum and sum (at most 64 shares)
+// grid (rows, heads, chunks of 64 value columns), one wave: lane sp holds share sp's maximum and sum (at most 64 shares) for the scale
+// factors; then lane = column, the shares' values read four at a time (independent requests, separate sums)
 __global__ void __launch_bounds__(64) k_attn_latent_rows_combine(LatRowArgs P)
 {
     const int t = blockIdx.x, h = blockIdx.y, dv = P.R, nsplit = P.nsplit, lane = threadIdx.x;
@@ -225,11 +226,17 @@ __global__ void __launch_bounds__(64) k_attn_latent_rows_combine(LatRowArgs P)
     const float M = wave_max(m_sp);
     const float f_sp = m_sp == -INFINITY ? 0.0f : expf(m_sp - M);
     const float L = wave_sum(l_sp * f_sp);
-    for (int d = lane; d < dv; d += 64) {
-        float o = 0.0f;
-        for (int sp = 0; sp < nsplit; sp++) o = fmaf(src[(size_t)sp * (dv + 2) + 2 + d], __shfl(f_sp, sp, 64), o);
-        P.out[(size_t)t * P.ldo + (size_t)h * dv + d] = o / L;
+    const int d = blockIdx.z * 64 + lane;
+    const float *col = src + 2 + min(d, dv - 1);
+    float o0 = 0.0f, o1 = 0.0f, o2 = 0.0f, o3 = 0.0f;
+    int sp = 0;
+    for (; sp + 4 <= nsplit; sp += 4) {
+        const float v0 = col[(size_t)sp * (dv + 2)], v1 = col[(size_t)(sp + 1) * (dv + 2)], v2 = col[(size_t)(sp + 2) * (dv + 2)], v3 = col[(size_t)(sp + 3) * (dv + 2)];
+        o0 = fmaf(v0, __shfl(f_sp, sp, 64), o0); o1 = fmaf(v1, __shfl(f_sp, sp + 1, 64), o1);
+        o2 = fmaf(v2, __shfl(f_sp, sp + 2, 64), o2); o3 = fmaf(v3, __shfl(f_sp, sp + 3, 64), o3);
     }
+    for (; sp < nsplit; sp++) o0 = fmaf(col[(size_t)sp * (dv + 2)], __shfl(f_sp, sp, 64), o0);
+    if (d < dv) P.out[(size_t)t * P.ldo + (size_t)h * dv + d] = ((o0 + o1) + (o2 + o3)) / L;
 }
 
 constexpr int LR_HB = 4, LR_MAX_SPLITS = 64;
@@ -492,7 +499,7 @@ int ifa_attention_latent_rows_f32(const void *qa_f32, size_t ldqa, int heads, in
     else if (cpl <= 4) launch_latent_rows<4>(P, (unsigned)rows, s);
     else if (cpl <= 8) launch_latent_rows<8>(P, (unsigned)rows, s);
     else launch_latent_rows<16>(P, (unsigned)rows, s);
-    hipLaunchKernelGGL(k_attn_latent_rows_combine, dim3((unsigned)rows, (unsigned)heads), dim3(64), 0, s, P);
+    hipLaunchKernelGGL(k_attn_latent_rows_combine, dim3((unsigned)rows, (unsigned)heads, ifa_cdiv((size_t)kv_rank, 64)), dim3(64), 0, s, P);
     IFA_LAUNCH_CHECK();
     return IFA_OK;
 }

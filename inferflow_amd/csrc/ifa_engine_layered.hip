@@ -77,6 +77,7 @@ struct LayeredNet {
     // Measured slower than the separate launches at width 2048 (decode 1149 tok/s without, 1068 / 1083 / 1012 with bit 0 / bit 1 / both; every
     // wave repeats the element-wise work for its rows) and within 1 % at width 1024: off by default
     int opt_fuse_rows = 0;
+    int opt_fuse_post = 1;                 // POSTNORM layers, steps of at most 8 rows: norm-add, depth average, next input convolution and its tail in one launch
     float *attn_ws = nullptr; size_t attn_ws_bytes = 0;      // partial results of the windowed attention when a (row, head)'s keys are shared out
     int opt_attn_tile_min = 16;            // steps of at least this many rows run the windowed attention through the tiled kernel
     std::vector<ifa_seq_desc> seqs_host;   // the current step's sequences (the tiled attention's grid is sized from them)
@@ -259,8 +260,33 @@ int linear(ifa_model *m, const bf16_t *W, size_t N, size_t K, const float *A, si
     return ifa_linear_bf16w(W, N, K, A, lda, T, bias, mul, alpha, accumulate, m->lay->cfg.ops32, C, ldc, silu0, silu1, (ifa_stream)m->stream);
 }
 
-// one POSTNORM layer over T rows: x <- x + norm1(mixer(x + conv1(x))); x <- x + norm2(experts(x + conv2(x)))
-int run_postnorm_layer(ifa_model *m, LLayer &L, size_t li, size_t T, int nseq)
+// What lies between two sub-layers of a POSTNORM block: x += gnorm(sub) * norm_w; [depth average]; [h = x + conv(x), tail advanced].
+// Steps of a few rows run it as ONE launch (ifa_norm_add_conv_rows_f32), larger steps as the separate row-parallel ops.
+int post_step(ifa_model *m, size_t T, int nseq, bool fused, const float *sub, const void *norm_w, const LLayer *depth_of, size_t li, const void *conv_w, int taps,
+              size_t conv_off)
+{
+    LayeredNet *n = m->lay;
+    const ifa_layered_config &c = n->cfg;
+    const size_t W = (size_t)c.width, plane = n->scratch_rows * W;
+    ifa_stream s = (ifa_stream)m->stream;
+    void *const *slots = (void *const *)n->slot_base_dev;
+    int rc;
+    if (fused)
+        return ifa_norm_add_conv_rows_f32(n->x, T, W, sub, W, norm_w, c.norm_groups, c.eps, depth_of ? n->stack : nullptr, plane, (int)li + 2,
+                                          depth_of ? depth_of->T(IFA_LT_DWA).data : nullptr, conv_w, taps, n->seqs_dev, nseq, n->row_seq_dev, slots, conv_off, n->h, s);
+    if (sub && (rc = ifa_group_rmsnorm_f32(sub, W, T, W, c.norm_groups, norm_w, c.eps, 1, n->x, W, s))) return rc;
+    if (depth_of && (rc = ifa_depth_average_f32(n->x, T, W, n->stack, plane, (int)li + 2, depth_of->T(IFA_LT_DWA).data, s))) return rc;
+    if (conv_w) {
+        if ((rc = ifa_shortconv_residual_f32(n->x, W, (int)W, taps, conv_w, n->seqs_dev, n->row_seq_dev, T, slots, conv_off, n->h, W, s))) return rc;
+        if ((rc = ifa_shortconv_tail_f32(n->x, W, (int)W, taps, n->seqs_dev, nseq, slots, conv_off, s))) return rc;
+    }
+    return IFA_OK;
+}
+
+// one POSTNORM layer over T rows: x <- x + norm1(mixer(x + conv1(x))); x <- x + norm2(experts(x + conv2(x))); depth average.
+// h_ready: the layer before has already left x + conv1(x) in n->h (its closing step ran this layer's input convolution);
+// next: the layer after, whose input convolution this layer's closing step runs when both are wired alike (*next_h_ready says so).
+int run_postnorm_layer(ifa_model *m, LLayer &L, size_t li, size_t T, int nseq, bool h_ready, const LLayer *next, bool *next_h_ready)
 {
     LayeredNet *n = m->lay;
     const ifa_layered_config &c = n->cfg;
@@ -268,12 +294,15 @@ int run_postnorm_layer(ifa_model *m, LLayer &L, size_t li, size_t T, int nseq)
     const size_t W = (size_t)c.width, NI = L.n_in;
     ifa_stream s = (ifa_stream)m->stream;
     void *const *slots = (void *const *)n->slot_base_dev;
+    const bool fused = T <= 8 && n->opt_fuse_post && !n->opt_tap_layers;
+    const bool moe = has_moe(sp);
+    const bool next_conv = fused && next && next->spec.block == IFA_BLOCK_POSTNORM && next->spec.canon_taps > 0;
+    *next_h_ready = next_conv;
     int rc;
     // what the mixer reads
     const float *hin = n->x;
     if (sp.canon_taps > 0) {
-        if ((rc = ifa_shortconv_residual_f32(n->x, W, (int)W, sp.canon_taps, L.T(IFA_LT_CANON1).data, n->seqs_dev, n->row_seq_dev, T, slots, L.o_cv1, n->h, W, s))) return rc;
-        if ((rc = ifa_shortconv_tail_f32(n->x, W, (int)W, sp.canon_taps, n->seqs_dev, nseq, slots, L.o_cv1, s))) return rc;
+        if (!h_ready && (rc = post_step(m, T, nseq, fused, nullptr, nullptr, nullptr, li, L.T(IFA_LT_CANON1).data, sp.canon_taps, L.o_cv1))) return rc;
         hin = n->h;
     }
     {   // latent attention
@@ -311,23 +340,27 @@ int run_postnorm_layer(ifa_model *m, LLayer &L, size_t li, size_t T, int nseq)
             if ((rc = ifa_latent_expand_out_f32(n->m4, (size_t)H * R, R, H, dv, R, L.T(IFA_LT_M_UV).data, gate, NI, T, n->m5, OV, s))) return rc;
         }
         if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_M_O).data, W, OV, n->m5, OV, T, nullptr, nullptr, 1.0f, 0, n->m1, W))) return rc;
-        if ((rc = ifa_group_rmsnorm_f32(n->m1, W, T, W, c.norm_groups, L.T(IFA_LT_NORM1).data, c.eps, 1, n->x, W, s))) return rc;
     }
-    if (has_moe(sp)) {
-        hin = n->x;
-        if (sp.canon_taps > 0) {
-            if ((rc = ifa_shortconv_residual_f32(n->x, W, (int)W, sp.canon_taps, L.T(IFA_LT_CANON2).data, n->seqs_dev, n->row_seq_dev, T, slots, L.o_cv2, n->h, W, s))) return rc;
-            if ((rc = ifa_shortconv_tail_f32(n->x, W, (int)W, sp.canon_taps, n->seqs_dev, nseq, slots, L.o_cv2, s))) return rc;
-            hin = n->h;
-        }
+    const LLayer *depth_of = sp.depth_avg ? &L : nullptr;
+    const void *ncw = next_conv ? next->T(IFA_LT_CANON1).data : nullptr;
+    const int ntaps = next_conv ? next->spec.canon_taps : 0;
+    const size_t noff = next_conv ? next->o_cv1 : 0;
+    if (!moe) return post_step(m, T, nseq, fused, n->m1, L.T(IFA_LT_NORM1).data, depth_of, li, ncw, ntaps, noff);
+    {
+        // the mixer's output into the residual, then what the experts read
+        if ((rc = post_step(m, T, nseq, fused, n->m1, L.T(IFA_LT_NORM1).data, nullptr, li, sp.canon_taps > 0 ? L.T(IFA_LT_CANON2).data : nullptr, sp.canon_taps, L.o_cv2))) return rc;
+        hin = sp.canon_taps > 0 ? n->h : n->x;
         const size_t XA = (size_t)(sp.x_experts + sp.x_identity);
-        if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_X_ROUTER).data, XA, W, hin, W, T, nullptr, nullptr, 1.0f, 0, n->m2, XA))) return rc;
-        if ((rc = ifa_moe_route_f32(n->m2, XA, T, (int)XA, sp.x_top, L.T(IFA_LT_X_CORR).data, n->moe_idx, n->moe_wgt, s))) return rc;
+        if (fused && XA <= 512) {      // a few rows: the router's product inside the choice's launch
+            if ((rc = ifa_moe_route_rows_f32(hin, W, T, (int)W, L.T(IFA_LT_X_ROUTER).data, (int)XA, sp.x_top, L.T(IFA_LT_X_CORR).data, n->moe_idx, n->moe_wgt, s))) return rc;
+        } else {
+            if ((rc = linear(m, (const bf16_t *)L.T(IFA_LT_X_ROUTER).data, XA, W, hin, W, T, nullptr, nullptr, 1.0f, 0, n->m2, XA))) return rc;
+            if ((rc = ifa_moe_route_f32(n->m2, XA, T, (int)XA, sp.x_top, L.T(IFA_LT_X_CORR).data, n->moe_idx, n->moe_wgt, s))) return rc;
+        }
         if ((rc = ifa_moe_experts_f32(hin, W, T, (int)W, std::max(sp.x_ff, 1), sp.x_experts, sp.x_identity, sp.x_top, 0, L.T(IFA_LT_X_UP).data, L.T(IFA_LT_X_DOWN).data,
                                       n->moe_idx, n->moe_wgt, c.ops32, n->moe_ws, n->moe_ws_bytes, n->m1, W, 0, s))) return rc;
-        if ((rc = ifa_group_rmsnorm_f32(n->m1, W, T, W, c.norm_groups, L.T(IFA_LT_NORM2).data, c.eps, 1, n->x, W, s))) return rc;
     }
-    return IFA_OK;
+    return post_step(m, T, nseq, fused, n->m1, L.T(IFA_LT_NORM2).data, depth_of, li, ncw, ntaps, noff);
 }
 
 // the layers of one step over T rows / nseq sequences whose tables are already on the device; leaves the residual in n->x
@@ -339,18 +372,19 @@ int run_layers(ifa_model *m, size_t T, int nseq)
     ifa_stream s = (ifa_stream)m->stream;
     void *const *slots = (void *const *)n->slot_base_dev;
     int rc;
-    const size_t plane = n->scratch_rows * W;          // one plane of the depth average
     if (c.stem == 1) {
         if ((rc = ifa_embed_rows_f32(n->embd.data, c.vocab, c.width, n->tokens_dev, T, n->h, s))) return rc;
         if ((rc = ifa_group_rmsnorm_f32(n->h, W, T, W, c.norm_groups, n->embd_norm.data, c.eps, 0, n->x, W, s))) return rc;
         if (n->any_depth_avg && (rc = ifa_group_rmsnorm_f32(n->h, W, T, W, c.norm_groups, n->embd_norm.data, c.eps, 0, n->stack, W, s))) return rc;      // plane 0
     } else if ((rc = ifa_embed_sinpos_f32(n->embd.data, c.vocab, c.width, n->tokens_dev, n->pos_dev, T, c.pos_base, n->x, s))) return rc;
+    bool h_ready = false;
     for (size_t li = 0; li < n->layers.size(); li++) {
         LLayer &L = n->layers[li];
         const ifa_layer_spec &sp = L.spec;
         if (sp.block == IFA_BLOCK_POSTNORM) {
-            if ((rc = run_postnorm_layer(m, L, li, T, nseq))) return rc;
-            if (sp.depth_avg && (rc = ifa_depth_average_f32(n->x, T, W, n->stack, plane, (int)li + 2, L.T(IFA_LT_DWA).data, s))) return rc;
+            bool next_ready = false;
+            if ((rc = run_postnorm_layer(m, L, li, T, nseq, h_ready, li + 1 < n->layers.size() ? &n->layers[li + 1] : nullptr, &next_ready))) return rc;
+            h_ready = next_ready;
             if (n->opt_tap_layers && n->taps && T <= n->taps_rows)
                 IFA_HIP_CHECK(hipMemcpyAsync(n->taps + li * n->taps_rows * W, n->x, T * W * 4, hipMemcpyDeviceToDevice, m->stream));
             continue;
@@ -636,10 +670,11 @@ int lay_set_option(ifa_model *m, const char *name, int value)
     LayeredNet *n = m->lay;
     if (!strcmp(name, "tap_layers")) { n->opt_tap_layers = value; drop_step_graph(n); return IFA_OK; }
     if (!strcmp(name, "fuse_rows")) { n->opt_fuse_rows = value; drop_step_graph(n); return IFA_OK; }
+    if (!strcmp(name, "fuse_post")) { n->opt_fuse_post = value; drop_step_graph(n); return IFA_OK; }
     if (!strcmp(name, "attn_tile_min")) { n->opt_attn_tile_min = value; return IFA_OK; }
     if (!strcmp(name, "graph")) { n->opt_graph = value; drop_step_graph(n); return IFA_OK; }
     if (!strcmp(name, "ops32")) { IFA_HIP_CHECK(hipStreamSynchronize(m->stream)); n->cfg.ops32 = value ? 1 : 0; drop_step_graph(n); return IFA_OK; }
-    return ifa_fail(IFA_ERR_ARG, "ifa_model_set_option: unknown option '%s' (layer-list model: tap_layers, graph, ops32, attn_tile_min, fuse_rows)", name);
+    return ifa_fail(IFA_ERR_ARG, "ifa_model_set_option: unknown option '%s' (layer-list model: tap_layers, graph, ops32, attn_tile_min, fuse_rows, fuse_post)", name);
 }
 
 int lay_set_excluded(ifa_model *m, const int *ids_host, int cnt)

@@ -48,6 +48,59 @@ __global__ void __launch_bounds__(64) k_moe_route(const float *__restrict__ logi
     }
 }
 
+// Steps of a few rows: the router's product and its choice in one launch.  A workgroup per row: the waves share out the router's outputs
+// (a dot of `width` each), then the scores and the `top` rounds as in k_moe_route (wave 0; the other waves only keep the barriers).
+__global__ void __launch_bounds__(1024) k_moe_route_rows(const float *__restrict__ h, size_t ldh, int W, const bf16_t *__restrict__ router, int n_all, int top,
+                                                        const bf16_t *__restrict__ corr, int *__restrict__ idx, float *__restrict__ wgt, int vec)
+{
+    extern __shared__ float sc[];          // [n_all] logits, then scores; [n_all] choice scores
+    float *ch = sc + n_all;
+    const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    const float *hr = h + (size_t)t * ldh;
+    for (int e = wave; e < n_all; e += nw) {
+        const bf16_t *w = router + (size_t)e * W;
+        float acc = 0.0f;
+        if (vec) {
+#pragma unroll 4
+            for (int k = lane * 8; k < W; k += 512) {
+                const u32x4m wv = *reinterpret_cast<const u32x4m *>(w + k);
+                const float4 a0 = *reinterpret_cast<const float4 *>(hr + k), a1 = *reinterpret_cast<const float4 *>(hr + k + 4);
+                acc = fmaf(a0.x, __uint_as_float(wv[0] << 16), acc); acc = fmaf(a0.y, __uint_as_float(wv[0] & 0xFFFF0000u), acc);
+                acc = fmaf(a0.z, __uint_as_float(wv[1] << 16), acc); acc = fmaf(a0.w, __uint_as_float(wv[1] & 0xFFFF0000u), acc);
+                acc = fmaf(a1.x, __uint_as_float(wv[2] << 16), acc); acc = fmaf(a1.y, __uint_as_float(wv[2] & 0xFFFF0000u), acc);
+                acc = fmaf(a1.z, __uint_as_float(wv[3] << 16), acc); acc = fmaf(a1.w, __uint_as_float(wv[3] & 0xFFFF0000u), acc);
+            }
+        } else {
+            for (int k = lane; k < W; k += 64) acc = fmaf(hr[k], bf2f(w[k]), acc);
+        }
+        acc = wave_sum(acc);
+        if (lane == 0) sc[e] = acc;
+    }
+    __syncthreads();
+    if (wave == 0) {
+        float mx = -INFINITY;
+        for (int e = lane; e < n_all; e += 64) mx = fmaxf(mx, sc[e]);
+        mx = wave_max(mx);
+        float sum = 0.0f;
+        for (int e = lane; e < n_all; e += 64) { const float pe = expf(sc[e] - mx); sc[e] = pe; sum += pe; }      // (each lane touches its own entries only)
+        sum = wave_sum(sum);
+        for (int e = lane; e < n_all; e += 64) { const float sv = sc[e] / sum; sc[e] = sv; ch[e] = sv + (corr ? bf2f(corr[e]) : 0.0f); }
+    }
+    __syncthreads();
+    for (int k = 0; k < top; k++) {
+        if (wave == 0) {
+            float best = -INFINITY; int bi = 0x7FFFFFFF;
+            for (int e = lane; e < n_all; e += 64) { const float v = ch[e]; if (v > best || (v == best && e < bi)) { best = v; bi = e; } }
+            for (int o = 32; o > 0; o >>= 1) {
+                const float ov = __shfl_xor(best, o, 64); const int oi = __shfl_xor(bi, o, 64);
+                if (ov > best || (ov == best && oi < bi)) { best = ov; bi = oi; }
+            }
+            if (lane == 0) { idx[(size_t)t * top + k] = bi; wgt[(size_t)t * top + k] = sc[bi]; ch[bi] = -INFINITY; }
+        }
+        __syncthreads();
+    }
+}
+
 // grid (ff chunks, pairs): act[p][n] = gelu(W_up[e][n] . h[t]); a wave per n at a time.  Identity pairs do nothing.
 __global__ void __launch_bounds__(256) k_moe_up_rows(const float *__restrict__ h, size_t ldh, int W, int F, int experts, int top, const bf16_t *__restrict__ up,
                                                      const int *__restrict__ idx, float *__restrict__ act, int vec)
@@ -194,6 +247,18 @@ int ifa_moe_route_f32(const void *logits_f32, size_t ld, size_t rows, int n_all,
     IFA_REQUIRE(rows > 0 && n_all >= 1 && n_all <= 4096 && top >= 1 && top <= n_all && ld >= (size_t)n_all, "ifa_moe_route_f32: bad shape (%d router outputs, %d chosen)", n_all, top);
     hipLaunchKernelGGL(k_moe_route, dim3((unsigned)rows), dim3(64), (size_t)n_all * 8, ifa_s(stream), (const float *)logits_f32, ld, n_all, top,
                        (const bf16_t *)correction_bf16, idx_dev, (float *)wgt_f32);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_moe_route_rows_f32(const void *h_f32, size_t ldh, size_t rows, int width, const void *router_bf16, int n_all, int top, const void *correction_bf16,
+                           int *idx_dev, void *wgt_f32, ifa_stream stream)
+{
+    IFA_REQUIRE(h_f32 && router_bf16 && idx_dev && wgt_f32, "ifa_moe_route_rows_f32: null pointer");
+    IFA_REQUIRE(rows > 0 && rows <= 64 && width > 0 && n_all >= 1 && n_all <= 4096 && top >= 1 && top <= n_all && ldh >= (size_t)width, "ifa_moe_route_rows_f32: bad shape");
+    const int vec = (width % 8 == 0 && ldh % 4 == 0 && ((uintptr_t)h_f32 & 15) == 0 && ((uintptr_t)router_bf16 & 15) == 0) ? 1 : 0;
+    hipLaunchKernelGGL(k_moe_route_rows, dim3((unsigned)rows), dim3(n_all > 8 ? 1024 : 256), (size_t)n_all * 8, ifa_s(stream), (const float *)h_f32, ldh, width,
+                       (const bf16_t *)router_bf16, n_all, top, (const bf16_t *)correction_bf16, idx_dev, (float *)wgt_f32, vec);
     IFA_LAUNCH_CHECK();
     return IFA_OK;
 }

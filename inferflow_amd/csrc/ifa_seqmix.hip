@@ -79,6 +79,78 @@ __global__ void __launch_bounds__(256) k_shortconv_residual(const float *__restr
     }
 }
 
+// Steps of a few rows: what lies between two sub-layers of a post-norm block in one launch --
+//   1. x[t] += m[t] / sqrt(mean_part(m[t]^2) + eps) * nw          (grouped RMS norm of a sub-layer's output into the residual; m null: skip)
+//   2. stack[count - 1] <- x; x <- sum_j dw[j] stack[j]            (depth average; stack null: skip)
+//   3. h[t] = x[t] + conv(x)[t]                                    (input convolution of the next sub-layer; cw null: skip)
+//   4. the convolution's carried tail advanced past the step's rows
+// A workgroup per norm part: stages 2 to 4 work channel by channel, stage 1 within a part, so a part's channels [c_lo, c_hi) never
+// meet another part's and the barriers between the stages are the workgroup's own.
+__global__ void __launch_bounds__(256) k_norm_add_conv_rows(float *__restrict__ x, int T, int W, const float *__restrict__ m, size_t ldm, const bf16_t *__restrict__ nw,
+                                                            int groups, float eps, float *__restrict__ stack, size_t plane, int count, const bf16_t *__restrict__ dw,
+                                                            const bf16_t *__restrict__ cw, int taps, const SeqDesc *__restrict__ seqs, int nseq,
+                                                            const int *__restrict__ row_seq, float *const *__restrict__ slot_base, size_t state_off,
+                                                            float *__restrict__ h)
+{
+    __shared__ float red[17];
+    const int tid = threadIdx.x, gs = W / groups, c_lo = blockIdx.x * gs, c_hi = c_lo + gs;
+    if (m) {
+        for (int t = 0; t < T; t++) {
+            const float *mr = m + (size_t)t * ldm;
+            float q = 0.0f;
+            for (int c = c_lo + tid; c < c_hi; c += blockDim.x) q = fmaf(mr[c], mr[c], q);
+            const float rinv = 1.0f / sqrtf(block_sum(q, red) / (float)gs + eps);
+            for (int c = c_lo + tid; c < c_hi; c += blockDim.x) {
+                float v = mr[c] * rinv;
+                if (nw) v *= bf2f(nw[c]);
+                x[(size_t)t * W + c] += v;
+            }
+        }
+    }
+    // (from here on a thread only meets values of its own channels: what it wrote above it reads back itself)
+    if (stack) {
+        for (int t = 0; t < T; t++)
+            for (int c = c_lo + tid; c < c_hi; c += blockDim.x) {
+                const size_t i = (size_t)t * W + c;
+                const float cur = x[i];
+                stack[(size_t)(count - 1) * plane + i] = cur;
+                float s = 0.0f;
+                for (int j = 0; j + 1 < count; j++) s = fmaf(bf2f(dw[j]), stack[(size_t)j * plane + i], s);
+                x[i] = fmaf(bf2f(dw[count - 1]), cur, s);
+            }
+    }
+    if (!cw) return;
+    for (int t = 0; t < T; t++) {
+        const SeqDesc sd = seqs[row_seq[t]];
+        const int i = t - sd.row0;
+        const float *tail = sd.pos0 > 0 ? slot_base[sd.slot] + state_off : nullptr;
+        for (int c = c_lo + tid; c < c_hi; c += blockDim.x) {
+            float acc = 0.0f;
+            for (int j = 0; j < taps; j++) {
+                const int idx = i - (taps - 1) + j;
+                float v;
+                if (idx >= 0) v = x[(size_t)(sd.row0 + idx) * W + c];
+                else v = tail ? tail[(size_t)(taps - 1 + idx) * W + c] : 0.0f;
+                acc = fmaf(bf2f(cw[(size_t)c * taps + j]), v, acc);
+            }
+            h[(size_t)t * W + c] = x[(size_t)t * W + c] + acc;
+        }
+    }
+    const int keep = taps - 1;
+    for (int q = 0; q < nseq; q++) {
+        const SeqDesc sd = seqs[q];
+        float *tail = slot_base[sd.slot] + state_off;
+        for (int c = c_lo + tid; c < c_hi; c += blockDim.x)
+            for (int r = 0; r < keep; r++) {          // ascending r: a value read from the old tail lies above what was written so far
+                const int idx = sd.n - keep + r;
+                float v;
+                if (idx >= 0) v = x[(size_t)(sd.row0 + idx) * W + c];
+                else v = sd.pos0 > 0 ? tail[(size_t)(keep + idx) * W + c] : 0.0f;
+                tail[(size_t)r * W + c] = v;
+            }
+    }
+}
+
 // grid: one workgroup per sequence.  The carried tail becomes the last taps - 1 inputs of (old tail, this step's rows).
 __global__ void __launch_bounds__(256) k_shortconv_tail(const float *__restrict__ x, size_t ldx, int C, int taps, const SeqDesc *__restrict__ seqs,
                                                         float *const *__restrict__ slot_base, size_t state_off)
@@ -365,6 +437,26 @@ int ifa_shortconv_residual_f32(const void *x_f32, size_t ldx, int channels, int 
     IFA_REQUIRE(channels > 0 && taps >= 1 && taps <= 64 && rows > 0 && ldx >= (size_t)channels && ldy >= (size_t)channels, "ifa_shortconv_residual_f32: bad shape");
     hipLaunchKernelGGL(k_shortconv_residual, dim3((unsigned)rows, std::min(8u, ifa_cdiv((size_t)channels, 256))), dim3(256), 0, ifa_s(stream), (const float *)x_f32, ldx,
                        channels, taps, (const bf16_t *)w_bf16, (const SeqDesc *)seqs_dev, row_seq_dev, (float *const *)slot_base_dev, state_off, (float *)y_f32, ldy);
+    IFA_LAUNCH_CHECK();
+    return IFA_OK;
+}
+
+int ifa_norm_add_conv_rows_f32(void *x_f32, size_t rows, size_t cols, const void *m_f32, size_t ldm, const void *norm_w_bf16, int groups, float eps,
+                               void *stack_f32, size_t plane_stride, int count, const void *depth_w_bf16, const void *conv_w_bf16, int taps,
+                               const void *seqs_dev, int n_seqs, const int *row_seq_dev, void *const *slot_base_dev, size_t state_off, void *h_f32,
+                               ifa_stream stream)
+{
+    IFA_REQUIRE(x_f32 && rows > 0 && rows <= 64 && cols > 0 && rows * cols < (1u << 30), "ifa_norm_add_conv_rows_f32: bad shape (%zu rows: at most 64)", rows);
+    IFA_REQUIRE(!m_f32 || (groups >= 1 && cols % (size_t)groups == 0 && ldm >= cols), "ifa_norm_add_conv_rows_f32: bad norm");
+    IFA_REQUIRE(!stack_f32 || (depth_w_bf16 && count >= 1 && plane_stride >= rows * cols), "ifa_norm_add_conv_rows_f32: bad depth average");
+    IFA_REQUIRE(!conv_w_bf16 || (taps >= 1 && taps <= 64 && seqs_dev && n_seqs > 0 && row_seq_dev && slot_base_dev && h_f32 && h_f32 != x_f32),
+                "ifa_norm_add_conv_rows_f32: bad convolution");
+    // a workgroup per norm part; without a norm the channels are shared out the same way (up to 64 parts that divide the row)
+    int parts = groups;
+    if (!m_f32) { parts = 1; while (parts < 64 && cols % (size_t)(parts * 2) == 0 && cols / (size_t)(parts * 2) >= 64) parts *= 2; }
+    hipLaunchKernelGGL(k_norm_add_conv_rows, dim3((unsigned)parts), dim3(256), 0, ifa_s(stream), (float *)x_f32, (int)rows, (int)cols, (const float *)m_f32, ldm,
+                       (const bf16_t *)norm_w_bf16, parts, eps, (float *)stack_f32, plane_stride, count, (const bf16_t *)depth_w_bf16, (const bf16_t *)conv_w_bf16, taps,
+                       (const SeqDesc *)seqs_dev, n_seqs, row_seq_dev, (float *const *)slot_base_dev, state_off, (float *)h_f32);
     IFA_LAUNCH_CHECK();
     return IFA_OK;
 }

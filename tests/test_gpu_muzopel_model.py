@@ -126,6 +126,21 @@ def test_portions_and_token_by_token_equal_the_whole_prompt(tmp_path, sizes):
     eng.close()
 
 
+def test_small_steps_as_fused_launches_and_as_separate_ops_agree(tmp_path):
+    """steps of a few rows run norm-add / depth average / input convolution / tail as one launch and the router's product inside its choice;
+    with the option off they take the row-parallel ops of the larger steps"""
+    import inferflow_amd as ia
+    w = fx.random_weights(MIXED, 25)
+    toks = tokens_for(MIXED, 60, 26)
+    want = oracle_logits(MIXED, w, toks)
+    eng = engine_for(tmp_path, MIXED, w)
+    for fuse in (1, 0, 1):
+        ia.check(ia.lib().ifa_model_set_option(eng.worker(), b"fuse_post", fuse))
+        for sizes in ([33, 1], [3, 2], [8, 7, 1]):
+            assert fx.rel_err(run_portions(eng, toks, sizes), want).max() < TOL32, (fuse, sizes)
+    eng.close()
+
+
 @pytest.mark.parametrize("n", [1, 2, 3, 4])
 def test_first_tokens_of_a_sequence(tmp_path, n):
     """prompts no longer than the convolution's taps, whole and token by token, on a slot that held a longer sequence before"""

@@ -229,6 +229,56 @@ def test_router_scores_choices_and_ties(rows, n_all, top):
         assert gi[0].tolist() == list(range(top))
 
 
+@pytest.mark.parametrize("rows,W,n_all,top", [(1, 64, 18, 4), (8, 30, 5, 5), (3, 256, 130, 6)])
+def test_router_with_its_product_inside(rows, W, n_all, top):
+    rng = np.random.default_rng(rows + W)
+    h = rng.standard_normal((rows, W + 2)).astype(np.float32)
+    R = bf16_round(rng.standard_normal((n_all, W)) * 0.3)
+    corr = bf16_round(0.1 * rng.standard_normal(n_all))
+    L = capi()
+    idx = torch.zeros((rows, top), dtype=torch.int32, device="cuda"); wgt = torch.zeros((rows, top), dtype=torch.float32, device="cuda")
+    ia.check(L.ifa_moe_route_rows_f32(p(dev32(h)), W + 2, rows, W, p(devbf(R)), n_all, top, p(devbf(corr)), p(idx), p(wgt), None)); sync()
+    z = t64(h[:, :W]) @ t64(R).T
+    wi, ww = orc.route(z, t64(corr), top)
+    s = torch.softmax(z, -1).numpy()
+    gi, gw = idx.cpu().numpy(), wgt.cpu().numpy()
+    for t in range(rows):
+        ch = np.sort(s[t] + corr.astype(np.float64))[::-1]
+        if top == n_all or ch[top - 1] - ch[top] > 1e-5:
+            assert sorted(gi[t]) == sorted(wi[t].tolist()), t
+        assert np.abs(gw[t] - s[t][gi[t]]).max() < 1e-5
+
+
+def test_norm_add_depth_average_convolution_in_one_launch_equals_the_separate_ops():
+    rng = np.random.default_rng(8)
+    W, taps, groups, count = 48, 3, 4, 3
+    L = capi()
+    seqs = [(2, 5, 0), (1, 0, 1), (3, 1, 2)]          # continued, new, continued
+    sd, rs, rows = seq_tables(seqs)
+    cw, nw, dw = devbf(bf16_round(0.5 * rng.standard_normal((W, taps)))), devbf(bf16_round(1 + 0.2 * rng.standard_normal(W))), devbf(bf16_round(rng.standard_normal(count)))
+    x0 = rng.standard_normal((rows, W)).astype(np.float32); sub = rng.standard_normal((rows, W + 4)).astype(np.float32)
+    stack0 = rng.standard_normal((count, 8, W)).astype(np.float32)
+    tails = [rng.standard_normal(((taps - 1) * W + 4,)).astype(np.float32) for _ in range(3)]
+    res = []
+    for fused in (True, False):
+        slots = Slots(3, (taps - 1) * W + 4)
+        for i in range(3):
+            slots.mem[i].copy_(torch.from_numpy(tails[i]))
+        x, st, h = dev32(x0), dev32(stack0), torch.zeros((rows, W), dtype=torch.float32, device="cuda")
+        if fused:
+            ia.check(L.ifa_norm_add_conv_rows_f32(p(x), rows, W, p(dev32(sub)), W + 4, p(nw), groups, 1e-6, p(st), 8 * W, count, p(dw), p(cw), taps, p(sd), len(seqs), p(rs),
+                                                  p(slots.table), 0, p(h), None))
+        else:
+            ia.check(L.ifa_group_rmsnorm_f32(p(dev32(sub)), W + 4, rows, W, groups, p(nw), 1e-6, 1, p(x), W, None))
+            ia.check(L.ifa_depth_average_f32(p(x), rows, W, p(st), 8 * W, count, p(dw), None))
+            ia.check(L.ifa_shortconv_residual_f32(p(x), W, W, taps, p(cw), p(sd), p(rs), rows, p(slots.table), 0, p(h), W, None))
+            ia.check(L.ifa_shortconv_tail_f32(p(x), W, W, taps, p(sd), len(seqs), p(slots.table), 0, None))
+        sync()
+        res.append([x.cpu().numpy(), st.cpu().numpy(), h.cpu().numpy()] + [mm.cpu().numpy()[:(taps - 1) * W] for mm in slots.mem])
+    for a, b in zip(*res):
+        assert np.abs(a - b).max() < 1e-5
+
+
 @pytest.mark.parametrize("rows,W,F,E,I,top", [(1, 64, 32, 6, 2, 3), (8, 64, 32, 6, 2, 8), (9, 64, 32, 6, 2, 3), (200, 96, 40, 16, 2, 4), (130, 30, 7, 3, 0, 1), (33, 32, 16, 0, 3, 2),
                                                (70, 64, 24, 70, 3, 8)])
 def test_experts_row_form_and_grouped_form(rows, W, F, E, I, top):
