@@ -20,7 +20,7 @@ typedef uint32_t u32x4m __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ float gelu_erf_f(float z) { return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f)); }
 
-// one wave per row: softmax over n_all logits, then `top` rounds of argmax over score + correction (lowest index on ties)
+// one wave per row: softmax over n_all logits, then `top` passes of argmax over score + correction (lowest index on ties)
 __global__ void __launch_bounds__(64) k_moe_route(const float *__restrict__ logits, size_t ld, int n_all, int top, const bf16_t *__restrict__ corr,
                                                   int *__restrict__ idx, float *__restrict__ wgt)
 {
@@ -49,7 +49,7 @@ __global__ void __launch_bounds__(64) k_moe_route(const float *__restrict__ logi
 }
 
 // Steps of a few rows: the router's product and its choice in one launch.  A workgroup per row: the waves share out the router's outputs
-// (a dot of `width` each), then the scores and the `top` rounds as in k_moe_route (wave 0; the other waves only keep the barriers).
+// (a dot of `width` each), then the scores and the `top` passes as in k_moe_route (wave 0; the other waves only keep the barriers).
 __global__ void __launch_bounds__(1024) k_moe_route_rows(const float *__restrict__ h, size_t ldh, int W, const bf16_t *__restrict__ router, int n_all, int top,
                                                         const bf16_t *__restrict__ corr, int *__restrict__ idx, float *__restrict__ wgt, int vec)
 {

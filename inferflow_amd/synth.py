@@ -177,7 +177,7 @@ def muzopel_config(width=2048, blocks=2, vocab=32000, heads=16, dim=128, rot_dim
     two = {"type": "latent_attention_2", "mixer": {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "scale": scale,
                                                    "rot": {"base": 10000.0, "dims": rot_dim}}, "mlp": mlp}
     one = {"type": "latent_attention", "mixer": {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "q_rank": q_rank, "scale": scale,
-                                                 "rot": {"base": 10000.0, "dims": rot_dim, "scaling": {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0}}},
+                                                 "rot": {"base": 10000.0, "dims": rot_dim, "scaling": {"factor": 4.0, "original": 2048, "fast": 32.0, "slow": 1.0}}},
            "mlp": mlp}
     return {"architecture": "Muzopel", "width": width, "vocab": vocab, "norm": {"eps": 1e-6, "groups": groups}, "canon": {"taps": taps}, "logit_softcap": 30.0,
             "layers": [two, two, two, one] * blocks}

@@ -32,7 +32,7 @@ def latent2_layer(heads=4, dim=16, rot_dim=16, vdim=40, kv_rank=24, base=50000.0
             "mlp": moe() if mlp == "default" else mlp}
 
 
-def config(layers, width=64, vocab=97, eps=1e-6, groups=4, taps=3, softcap=12.0):
+def config(layers, width=64, vocab=97, eps=1e-6, groups=2, taps=4, softcap=12.0):
     return {"architecture": "Muzopel", "width": width, "vocab": vocab, "norm": {"eps": eps, "groups": groups}, "canon": {"taps": taps},
             "logit_softcap": softcap, "layers": layers}
 

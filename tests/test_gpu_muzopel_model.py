@@ -161,7 +161,7 @@ def test_batches_of_unequal_requests_equal_each_alone_and_slots_are_reused(tmp_p
     prompts = [tokens_for(MIXED, n, 10 + n) for n in (1, 37, 64, 5, 90, 2)]
     tails = [tokens_for(MIXED, 12, 50 + i) for i in range(len(prompts))]
     alone = [oracle_logits(MIXED, w, p + t) for p, t in zip(prompts, tails)]
-    # two rounds of three queries on three slots: the second round reuses the slots of the first
+    # three queries on three slots, twice: the second time reuses the slots of the first
     for rnd in range(2):
         qs = [eng.add_query(p) for p in prompts[3 * rnd:3 * rnd + 3]]
         assert all(q > 0 for q in qs) and eng.add_query([1, 2]) == 0          # busy: every slot is taken

@@ -61,11 +61,11 @@ def test_depth_average_that_keeps_only_the_newest_result_changes_nothing():
 
 
 def test_scaled_rotation_keeps_fast_pairs_and_slows_slow_pairs():
-    rot = {"base": 10000.0, "dims": 16, "scaling": {"factor": 8.0, "original": 1024, "fast": 32.0, "slow": 1.0}}
+    rot = {"base": 5000.0, "dims": 12, "scaling": {"factor": 4.0, "original": 512, "fast": 16.0, "slow": 2.0}}
     cos, sin = orc.rotation_tables(rot, 2)
-    mult = 0.1 * math.log(8.0) + 1.0
-    f = 10000.0 ** (-2.0 * np.arange(8) / 16)
+    mult = 0.1 * math.log(4.0) + 1.0
+    f = 5000.0 ** (-2.0 * np.arange(6) / 12)
     ang = np.arctan2(sin[1].numpy(), cos[1].numpy())
     assert np.allclose(np.hypot(cos[1].numpy(), sin[1].numpy()), mult)
-    assert np.isclose(ang[0], f[0]) and np.isclose(ang[-1], f[-1] / 8.0)       # the fastest pair is untouched, the slowest divided by the factor
-    assert np.all(ang <= f + 1e-12) and np.all(ang >= f / 8.0 - 1e-12)
+    assert np.isclose(ang[0], f[0]) and np.isclose(ang[-1], f[-1] / 4.0)       # the fastest pair is untouched, the slowest divided by the factor
+    assert np.all(ang <= f + 1e-12) and np.all(ang >= f / 4.0 - 1e-12)
