@@ -572,6 +572,9 @@ int ifa_latent_absorb_q_f32(const void *q_f32, size_t ldq, int heads, int dim, i
 int ifa_attention_latent_rows_f32(const void *qa_f32, size_t ldqa, int heads, int kv_rank, int rot_dim, float scale, const void *seqs_dev,
                                   const int *row_seq_dev, size_t rows, void *const *slot_base_dev, size_t cache_off, int max_keys, void *ws_f32,
                                   size_t ws_bytes, void *out_f32, size_t ldo, ifa_stream stream);
+/* asks ahead for the LDS the single-token kernel needs for this row shape (beyond 48 KB it has to be granted once per kernel): call it
+ * before a step that may be captured into a graph, where the grant cannot be asked for */
+int ifa_attention_latent_rows_reserve(int kv_rank, int rot_dim);
 /* out[t][h * vdim + e] = gate[t][h] * sum_r w_uv[h * vdim + e][r] * ol[t][h * ld_head + r]; gate = sigmoid(g[t][h]) or 1 (g null) */
 int ifa_latent_expand_out_f32(const void *ol_f32, size_t ldol, int ld_head, int heads, int vdim, int kv_rank, const void *w_uv_bf16,
                               const void *g_f32, size_t ldg, size_t rows, void *out_f32, size_t ldo, ifa_stream stream);

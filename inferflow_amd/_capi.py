@@ -172,6 +172,7 @@ SIGNATURES = {
     "ifa_latent_prepare_f32": (_i, [_vp, _sz, _i, _i, _i, _vp, _f, _vp, _sz, _i, _i, _vp, _f, _vp, _vp, _sz, _vp, _sz, _vp]),
     "ifa_latent_absorb_q_f32": (_i, [_vp, _sz, _i, _i, _i, _i, _vp, _sz, _vp, _sz, _vp]),
     "ifa_attention_latent_rows_f32": (_i, [_vp, _sz, _i, _i, _i, _f, _vp, _vp, _sz, _vp, _sz, _i, _vp, _sz, _vp, _sz, _vp]),
+    "ifa_attention_latent_rows_reserve": (_i, [_i, _i]),
     "ifa_latent_expand_out_f32": (_i, [_vp, _sz, _i, _i, _i, _i, _vp, _vp, _sz, _sz, _vp, _sz, _vp]),
     "ifa_attention_latent_tile_f32": (_i, [_vp, _sz, _i, _i, _i, _i, _i, _f, _vp, _sz, _vp, _sz, _vp, _vp, _sz, _vp, _vp, _i, _vp, _sz, _vp, _sz, _vp]),
     "ifa_attention_latent_tile_fits": (_i, [_i, _i, _i]),

@@ -241,12 +241,36 @@ __global__ void __launch_bounds__(64) k_attn_latent_rows_combine(LatRowArgs P)
 
 constexpr int LR_HB = 4, LR_MAX_SPLITS = 64;
 
+size_t latent_rows_smem(int R, int dr) { return ((size_t)LR_HB * (R + dr) + 8 * LR_HB + (size_t)4 * LR_HB * R) * 4; }
+
+// LDS beyond 48 KB has to be granted per kernel; `reserved` remembers the largest grant of this instantiation so that a launch
+// inside a captured step does not have to ask (ifa_attention_latent_rows_reserve asks ahead)
+template <int CPL>
+int reserve_latent_rows(size_t smem)
+{
+    static size_t reserved = 48 * 1024;
+    if (smem <= reserved) return IFA_OK;
+    IFA_REQUIRE(smem <= 160 * 1024, "ifa_attention_latent_rows_f32: %zu bytes of LDS", smem);
+    IFA_HIP_CHECK(hipFuncSetAttribute((const void *)k_attn_latent_rows<LR_HB, CPL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem));
+    reserved = smem;
+    return IFA_OK;
+}
+
+int reserve_latent_rows_for(int R, int dr)
+{
+    const int cpl = (R + 63) / 64;
+    const size_t smem = latent_rows_smem(R, dr);
+    if (cpl <= 1) return reserve_latent_rows<1>(smem);
+    if (cpl <= 2) return reserve_latent_rows<2>(smem);
+    if (cpl <= 4) return reserve_latent_rows<4>(smem);
+    if (cpl <= 8) return reserve_latent_rows<8>(smem);
+    return reserve_latent_rows<16>(smem);
+}
+
 template <int CPL>
 void launch_latent_rows(const LatRowArgs &P, unsigned rows, hipStream_t s)
 {
-    const size_t smem = ((size_t)LR_HB * (P.R + P.dr) + 8 * LR_HB + (size_t)4 * LR_HB * P.R) * 4;
-    if (smem > 48 * 1024) (void)hipFuncSetAttribute((const void *)k_attn_latent_rows<LR_HB, CPL>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
-    hipLaunchKernelGGL((k_attn_latent_rows<LR_HB, CPL>), dim3(rows, (unsigned)((P.heads + LR_HB - 1) / LR_HB), (unsigned)P.nsplit), dim3(256), smem, s, P);
+    hipLaunchKernelGGL((k_attn_latent_rows<LR_HB, CPL>), dim3(rows, (unsigned)((P.heads + LR_HB - 1) / LR_HB), (unsigned)P.nsplit), dim3(256), latent_rows_smem(P.R, P.dr), s, P);
 }
 
 // ---- prompts: 128 queries of one sequence per workgroup, the keys 0 .. last query walked in blocks of 32 staged once per workgroup in
@@ -493,6 +517,8 @@ int ifa_attention_latent_rows_f32(const void *qa_f32, size_t ldqa, int heads, in
     IFA_REQUIRE(rows * (size_t)heads * nsplit * ((size_t)kv_rank + 2) * 4 <= ws_bytes, "ifa_attention_latent_rows_f32: workspace of %zu bytes is too small", ws_bytes);
     P.nsplit = nsplit;
     hipStream_t s = ifa_s(stream);
+    int rc;
+    if ((rc = reserve_latent_rows_for(kv_rank, rot_dim))) return rc;
     const int cpl = (kv_rank + 63) / 64;
     if (cpl <= 1) launch_latent_rows<1>(P, (unsigned)rows, s);
     else if (cpl <= 2) launch_latent_rows<2>(P, (unsigned)rows, s);
@@ -502,6 +528,12 @@ int ifa_attention_latent_rows_f32(const void *qa_f32, size_t ldqa, int heads, in
     hipLaunchKernelGGL(k_attn_latent_rows_combine, dim3((unsigned)rows, (unsigned)heads, ifa_cdiv((size_t)kv_rank, 64)), dim3(64), 0, s, P);
     IFA_LAUNCH_CHECK();
     return IFA_OK;
+}
+
+int ifa_attention_latent_rows_reserve(int kv_rank, int rot_dim)
+{
+    IFA_REQUIRE(kv_rank > 0 && kv_rank <= 1024 && rot_dim >= 0, "ifa_attention_latent_rows_reserve: bad shape");
+    return reserve_latent_rows_for(kv_rank, rot_dim);
 }
 
 int ifa_attention_latent_tile_f32(const void *q_f32, size_t ldq, int heads, int dim, int rot_dim, int vdim, int kv_rank, float scale,

@@ -564,6 +564,7 @@ int lay_finalize(ifa_model *m)
             n->ffn_max = std::max(n->ffn_max, (size_t)sp.m_q_rank);
             n->kx_max = std::max(n->kx_max, H * (size_t)sp.m_dim); n->vx_max = std::max(n->vx_max, H * (size_t)sp.m_vdim);
             n->any_latent = true;
+            if ((rc = ifa_attention_latent_rows_reserve(sp.m_kv_rank, sp.m_rot_dim))) return rc;      // (the single-token step may be captured)
             if (!ifa_attention_latent_tile_fits(sp.m_dim, sp.m_rot_dim, sp.m_vdim)) n->latent_tile_ok = false;
             if (has_moe(sp)) {
                 if (sp.canon_taps > 1) { L.o_cv2 = off; off += align4((size_t)(sp.canon_taps - 1) * W); }

@@ -347,6 +347,25 @@ def test_greedy_generation_through_the_engine(tmp_path):
     eng.close()
 
 
+def test_generation_with_a_cache_row_that_needs_the_large_lds_grant(tmp_path):
+    """a latent of 640 channels: the single-token kernel's LDS passes 48 KB, granted when the model is finalized, before the step is captured"""
+    cfg = fx.config([fx.latent2_layer(heads=5, dim=16, rot_dim=16, vdim=24, kv_rank=640, mlp=fx.moe(experts=3, identity=1, top=2, ff=16))], width=32, vocab=37)
+    w = fx.random_weights(cfg, 41)
+    prompt = tokens_for(cfg, 21, 42)
+    eng = engine_for(tmp_path, cfg, w)
+    q = eng.add_query(prompt)
+    gen, _ = eng.generate(q, 12)
+    eng.remove_query(q)
+    want = oracle_logits(cfg, w, prompt + gen)
+    for i, tok in enumerate(gen):
+        row = want[len(prompt) - 1 + i]
+        top2 = np.sort(row)[-2:]
+        if top2[1] - top2[0] > 1e-3 * np.abs(row).max():
+            assert tok == int(row.argmax()), i
+    assert fx.rel_err(run_portions(eng, prompt + gen, [17, 1]), want).max() < TOL32
+    eng.close()
+
+
 def test_ini_route_and_trace_replay_tool(tmp_path):
     from inferflow_amd.engine import InferenceEngine
     w = fx.random_weights(MIXED, 17)
